@@ -1,0 +1,127 @@
+"""
+ctypes binding of `libfastmoe_hip.so` (C ABI declared in `include/fastmoe_hip.h`).
+
+The library is the only compute path of this package: if it is missing or a symbol is absent, importing this module
+raises. Build it with `python -m fast_llm_amd.build`.
+"""
+
+import ctypes
+import pathlib
+
+import torch
+
+LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "csrc" / "libfastmoe_hip.so"
+
+FM_VERSION = 1
+
+_c_i64, _c_int, _c_ptr, _c_size = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+
+# name -> (restype, argtypes). Mirrors include/fastmoe_hip.h one to one; tests check that every declared symbol
+# is listed here and exported by the library.
+SIGNATURES: dict[str, tuple] = {
+    "fm_version": (_c_int, []),
+    "fm_last_error": (ctypes.c_char_p, []),
+    "fm_sparse_map_workspace_size": (_c_size, [_c_i64] * 3),
+    "fm_sparse_map": (_c_int, [_c_ptr] + [_c_i64] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_size, _c_ptr]),
+    "fm_copy_dense_to_sparse": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int] * 3 + [_c_ptr]),
+    "fm_copy_sparse_to_dense": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int] * 3 + [_c_ptr]),
+    "fm_copy_sparse_to_dense_grad_score": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int] * 3 + [_c_ptr]),
+    "fm_copy_sparse_to_dense_backward": (_c_int, [_c_ptr] * 6 + [_c_i64] * 4 + [_c_int] * 4 + [_c_ptr]),
+    "fm_mlp_activation_forward": (_c_int, [_c_ptr] * 2 + [_c_i64] * 2 + [_c_int] * 3 + [_c_ptr]),
+    "fm_mlp_activation_backward": (_c_int, [_c_ptr] * 4 + [_c_i64] * 2 + [_c_int] * 3 + [_c_ptr]),
+    "fm_output_sparse_matmul": (_c_int, [_c_ptr] * 4 + [_c_i64] * 10 + [_c_int] * 4 + [_c_ptr]),
+    "fm_input_inner_sparse_matmul": (_c_int, [_c_ptr] * 4 + [_c_i64] * 10 + [_c_int] * 4 + [_c_ptr]),
+    "fm_input_row_sparse_matmul": (_c_int, [_c_ptr] * 5 + [_c_i64] * 10 + [_c_int] * 4 + [_c_ptr]),
+}
+
+FM_ERR_INVALID_ARGUMENT, FM_ERR_UNSUPPORTED, FM_ERR_LAUNCH = -1, -2, -3
+
+DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+INDEX_DTYPES = {torch.int16: 0, torch.int32: 1, torch.int64: 2}
+ACTIVATIONS = {"gelu": 0, "silu": 1, "relu": 2, "squared_relu": 3, "identity": 4}
+
+
+class FastMoeLibraryError(ImportError):
+    pass
+
+
+def load_library(path: pathlib.Path = LIBRARY_PATH) -> ctypes.CDLL:
+    if not path.is_file():
+        raise FastMoeLibraryError(
+            f"{path} is missing: the HIP kernel library is the only compute path of fast_llm_amd. "
+            "Build it with `python -m fast_llm_amd.build` (needs hipcc; no GPU required to compile)."
+        )
+    library = ctypes.CDLL(str(path))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        try:
+            function = getattr(library, name)
+        except AttributeError as e:
+            raise FastMoeLibraryError(f"{path} does not export `{name}`; rebuild it") from e
+        function.restype = restype
+        function.argtypes = argtypes
+    version = library.fm_version()
+    if version != FM_VERSION:
+        raise FastMoeLibraryError(f"{path} has ABI version {version}, this package needs {FM_VERSION}; rebuild it")
+    return library
+
+
+_library: ctypes.CDLL | None = None
+
+
+def lib() -> ctypes.CDLL:
+    global _library
+    if _library is None:
+        _library = load_library()
+    return _library
+
+
+def check(status: int) -> None:
+    """Turn a negative `fm_status` into the exception the reference's Python code would raise."""
+    if status == 0:
+        return
+    message = lib().fm_last_error().decode()
+    if status == FM_ERR_LAUNCH:
+        raise RuntimeError(message)
+    if status == FM_ERR_UNSUPPORTED:
+        raise NotImplementedError(message)
+    raise ValueError(message)
+
+
+def require_device(*tensors: torch.Tensor | None) -> torch.device:
+    """All tensors must live on one HIP device; there is no host implementation to fall back to."""
+    device = None
+    for tensor in tensors:
+        if tensor is None:
+            continue
+        if tensor.device.type != "cuda":
+            raise RuntimeError(
+                f"fast_llm_amd kernels run on the GPU only, got a tensor on `{tensor.device}` (there is no CPU path)"
+            )
+        if device is None:
+            device = tensor.device
+        elif tensor.device != device:
+            raise RuntimeError(f"tensors on different devices: {device} and {tensor.device}")
+    assert device is not None
+    return device
+
+
+def ptr(tensor: torch.Tensor | None) -> int | None:
+    return None if tensor is None else tensor.data_ptr()
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def dtype_tag(dtype: torch.dtype) -> int:
+    try:
+        return DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype} (supported: float32, bfloat16, float16)") from None
+
+
+def index_tag(dtype: torch.dtype) -> int:
+    try:
+        return INDEX_DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported index dtype {dtype} (supported: int16, int32, int64)") from None

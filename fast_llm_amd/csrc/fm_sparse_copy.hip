@@ -1,0 +1,322 @@
+// Bandwidth-bound gather/scatter between the dense token layout [T, H] and the expert-sorted sparse layout
+// [R, H]: dispatch (dense -> sparse), combine (sparse -> dense), the score gradient of the combine, and the
+// fused backward of the combine.
+//
+// One workgroup per token row. Every lane moves 16-byte vectors (8 bf16 / 4 fp32), consecutive lanes touch
+// consecutive vectors, so each wavefront access is one contiguous 1 KiB segment of a row. The k row indices
+// and scores of a token are wave-uniform and live in scalar registers. Rows whose index is negative are
+// skipped (the sparse map marks out-of-range experts that way).
+//
+// Arithmetic contract (reference: fast_llm/functional/triton/sparse_copy.py:27-49, 69-90, 111-148):
+// products and sums in fp32, scores converted to fp32 on load, one rounding at the store, combine adds the
+// slots in the order j = 0 .. k-1.
+#include "fm_common.h"
+
+namespace fm {
+
+constexpr int kCopyThreads = 256;
+
+struct CopyArgs {
+    const void *sparse_rows;
+    const void *scores;  // may be null
+    int64_t num_columns;
+    int experts_per_token;
+    int index_dtype;
+    int scores_dtype;
+};
+
+__device__ __forceinline__ float load_score(const void *scores, int scores_dtype, int64_t i) {
+    if (scores_dtype == FM_DTYPE_F32) return static_cast<const float *>(scores)[i];
+    if (scores_dtype == FM_DTYPE_BF16) return to_float(static_cast<const bf16_t *>(scores)[i]);
+    return to_float(static_cast<const f16_t *>(scores)[i]);
+}
+
+// ---- dispatch ------------------------------------------------------------------------------------------
+template <typename T, bool kVector>
+__global__ __launch_bounds__(kCopyThreads) void copy_dense_to_sparse_kernel(const T *__restrict__ input,
+                                                                            T *__restrict__ output, CopyArgs args) {
+    constexpr int N = kVector ? Vec16<T>::N : 1;
+    const int64_t token = blockIdx.x;
+    const int64_t columns = args.num_columns;
+    const T *in_row = input + token * columns;
+    const int k = args.experts_per_token;
+    for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns; c += static_cast<int64_t>(blockDim.x) * N) {
+        Vec16<T> value;
+        if constexpr (kVector) value = load16(in_row + c);
+        else value.v[0] = in_row[c];
+        for (int j = 0; j < k; ++j) {
+            const int64_t row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
+            if (row < 0) continue;
+            Vec16<T> scaled = value;
+            if (args.scores != nullptr) {
+                const float score = load_score(args.scores, args.scores_dtype, token * k + j);
+#pragma unroll
+                for (int i = 0; i < N; ++i) scaled.v[i] = from_float<T>(to_float(value.v[i]) * score);
+            }
+            if constexpr (kVector) store16(output + row * columns + c, scaled);
+            else output[row * columns + c] = scaled.v[0];
+        }
+    }
+}
+
+// ---- combine -------------------------------------------------------------------------------------------
+template <typename T, bool kVector>
+__global__ __launch_bounds__(kCopyThreads) void copy_sparse_to_dense_kernel(const T *__restrict__ input,
+                                                                            T *__restrict__ output, CopyArgs args) {
+    constexpr int N = kVector ? Vec16<T>::N : 1;
+    const int64_t token = blockIdx.x;
+    const int64_t columns = args.num_columns;
+    const int k = args.experts_per_token;
+    for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns; c += static_cast<int64_t>(blockDim.x) * N) {
+        float sum[N];
+#pragma unroll
+        for (int i = 0; i < N; ++i) sum[i] = 0.f;
+        for (int j = 0; j < k; ++j) {
+            const int64_t row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
+            if (row < 0) continue;
+            Vec16<T> value;
+            if constexpr (kVector) value = load16(input + row * columns + c);
+            else value.v[0] = input[row * columns + c];
+            if (args.scores != nullptr) {
+                const float score = load_score(args.scores, args.scores_dtype, token * k + j);
+#pragma unroll
+                for (int i = 0; i < N; ++i) sum[i] += to_float(value.v[i]) * score;
+            } else {
+#pragma unroll
+                for (int i = 0; i < N; ++i) sum[i] += to_float(value.v[i]);
+            }
+        }
+        Vec16<T> result;
+#pragma unroll
+        for (int i = 0; i < N; ++i) result.v[i] = from_float<T>(sum[i]);
+        if constexpr (kVector) store16(output + token * columns + c, result);
+        else output[token * columns + c] = result.v[0];
+    }
+}
+
+// ---- score gradient, optionally fused with the scaled dispatch of grad_output ---------------------------
+// grad_scores[t, j] = <input[row(t, j), :], grad_output[t, :]>; when kFused also
+// grad_input[row(t, j), :] = grad_output[t, :] * scores[t, j].
+// kChunks vectors of grad_output per lane are kept in registers across the k slots.
+template <typename T, typename OutT, bool kVector, bool kFused, int kChunks>
+__global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__restrict__ input,
+                                                                  const T *__restrict__ grad_output,
+                                                                  T *__restrict__ grad_input,
+                                                                  OutT *__restrict__ grad_scores, CopyArgs args) {
+    constexpr int N = kVector ? Vec16<T>::N : 1;
+    __shared__ float lds_partial[kCopyThreads / 64];
+    const int64_t token = blockIdx.x;
+    const int64_t columns = args.num_columns;
+    const int k = args.experts_per_token;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const T *grad_row = grad_output + token * columns;
+
+    Vec16<T> grad[kChunks > 0 ? kChunks : 1];
+    if constexpr (kChunks > 0) {
+#pragma unroll
+        for (int q = 0; q < kChunks; ++q) {
+            const int64_t c = (static_cast<int64_t>(q) * blockDim.x + threadIdx.x) * N;
+            if (c < columns) {
+                if constexpr (kVector) grad[q] = load16(grad_row + c);
+                else grad[q].v[0] = grad_row[c];
+            }
+        }
+    }
+
+    for (int j = 0; j < k; ++j) {
+        const int64_t row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
+        float score = 0.f;
+        if constexpr (kFused) score = load_score(args.scores, args.scores_dtype, token * k + j);
+        float partial = 0.f;
+        if (row >= 0) {
+            const T *in_row = input + row * columns;
+            T *out_row = kFused ? grad_input + row * columns : nullptr;
+            auto body = [&](const Vec16<T> &g, int64_t c) {
+                Vec16<T> value;
+                if constexpr (kVector) value = load16(in_row + c);
+                else value.v[0] = in_row[c];
+#pragma unroll
+                for (int i = 0; i < N; ++i) partial += to_float(value.v[i]) * to_float(g.v[i]);
+                if constexpr (kFused) {
+                    Vec16<T> scaled;
+#pragma unroll
+                    for (int i = 0; i < N; ++i) scaled.v[i] = from_float<T>(to_float(g.v[i]) * score);
+                    if constexpr (kVector) store16(out_row + c, scaled);
+                    else out_row[c] = scaled.v[0];
+                }
+            };
+            if constexpr (kChunks > 0) {
+#pragma unroll
+                for (int q = 0; q < kChunks; ++q) {
+                    const int64_t c = (static_cast<int64_t>(q) * blockDim.x + threadIdx.x) * N;
+                    if (c < columns) body(grad[q], c);
+                }
+            } else {
+                for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns;
+                     c += static_cast<int64_t>(blockDim.x) * N) {
+                    Vec16<T> g;
+                    if constexpr (kVector) g = load16(grad_row + c);
+                    else g.v[0] = grad_row[c];
+                    body(g, c);
+                }
+            }
+        }
+        partial = wave_sum(partial);
+        if (lane == 0) lds_partial[wave] = partial;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float total = 0.f;
+            for (int w = 0; w < waves; ++w) total += lds_partial[w];
+            grad_scores[token * k + j] = from_float<OutT>(total);
+        }
+        __syncthreads();
+    }
+}
+
+static int copy_threads(int64_t num_columns, int vector) {
+    const int64_t chunks = (num_columns + vector - 1) / vector;
+    int64_t threads = (chunks + 63) / 64 * 64;
+    if (threads > kCopyThreads) threads = kCopyThreads;
+    if (threads < 64) threads = 64;
+    return static_cast<int>(threads);
+}
+
+static int validate_copy(const char *name, const void *a, const void *b, const void *sparse_rows, int64_t rows,
+                         int64_t columns, int64_t k, int64_t rows_sparse, int dtype, int scores_dtype,
+                         int index_dtype) {
+    FM_REQUIRE(rows >= 0 && columns >= 0 && k >= 0 && rows_sparse >= 0, "%s: negative shape", name);
+    FM_REQUIRE(rows < (int64_t(1) << 31), "%s: too many rows", name);
+    FM_REQUIRE(valid_dtype(dtype) && valid_dtype(scores_dtype), "%s: bad dtype", name);
+    FM_REQUIRE(valid_index_dtype(index_dtype), "%s: bad index_dtype %d", name, index_dtype);
+    FM_REQUIRE(rows == 0 || columns == 0 || (a && b), "%s: null tensor", name);
+    FM_REQUIRE(rows == 0 || k == 0 || sparse_rows, "%s: null sparse_rows", name);
+    return FM_OK;
+}
+
+}  // namespace fm
+
+using namespace fm;
+
+extern "C" int fm_copy_dense_to_sparse(const void *input, const void *scores, const void *sparse_rows, void *output,
+                                       int64_t num_rows_dense, int64_t num_columns, int64_t num_experts_per_token,
+                                       int64_t num_rows_sparse, int dtype, int scores_dtype, int index_dtype,
+                                       void *stream_) {
+    const char *name = "fm_copy_dense_to_sparse";
+    if (int status = validate_copy(name, input, output, sparse_rows, num_rows_dense, num_columns,
+                                   num_experts_per_token, num_rows_sparse, dtype, scores_dtype, index_dtype))
+        return status;
+    if (num_rows_dense == 0 || num_columns == 0 || num_experts_per_token == 0) return FM_OK;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    CopyArgs args{sparse_rows, scores, num_columns, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype};
+    const int vector = 16 / dtype_size(dtype);
+    const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(output);
+    const int threads = copy_threads(num_columns, vectorised ? vector : 1);
+    FM_DISPATCH_DTYPE(dtype, T, {
+        if (vectorised)
+            copy_dense_to_sparse_kernel<T, true><<<num_rows_dense, threads, 0, stream>>>(
+                static_cast<const T *>(input), static_cast<T *>(output), args);
+        else
+            copy_dense_to_sparse_kernel<T, false><<<num_rows_dense, threads, 0, stream>>>(
+                static_cast<const T *>(input), static_cast<T *>(output), args);
+    });
+    return check_launch(name);
+}
+
+extern "C" int fm_copy_sparse_to_dense(const void *input, const void *scores, const void *sparse_rows, void *output,
+                                       int64_t num_rows_dense, int64_t num_columns, int64_t num_experts_per_token,
+                                       int64_t num_rows_sparse, int dtype, int scores_dtype, int index_dtype,
+                                       void *stream_) {
+    const char *name = "fm_copy_sparse_to_dense";
+    if (int status = validate_copy(name, num_experts_per_token ? input : output, output, sparse_rows, num_rows_dense,
+                                   num_columns, num_experts_per_token, num_rows_sparse, dtype, scores_dtype,
+                                   index_dtype))
+        return status;
+    if (num_rows_dense == 0 || num_columns == 0) return FM_OK;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    CopyArgs args{sparse_rows, scores, num_columns, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype};
+    const int vector = 16 / dtype_size(dtype);
+    const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(output);
+    const int threads = copy_threads(num_columns, vectorised ? vector : 1);
+    FM_DISPATCH_DTYPE(dtype, T, {
+        if (vectorised)
+            copy_sparse_to_dense_kernel<T, true><<<num_rows_dense, threads, 0, stream>>>(
+                static_cast<const T *>(input), static_cast<T *>(output), args);
+        else
+            copy_sparse_to_dense_kernel<T, false><<<num_rows_dense, threads, 0, stream>>>(
+                static_cast<const T *>(input), static_cast<T *>(output), args);
+    });
+    return check_launch(name);
+}
+
+namespace fm {
+
+template <typename T, typename OutT, bool kFused>
+static void launch_grad_score(const void *input, const void *grad_output, void *grad_input, void *grad_scores,
+                              int64_t rows, const CopyArgs &args, bool vectorised, int threads, hipStream_t stream) {
+    const T *in = static_cast<const T *>(input);
+    const T *go = static_cast<const T *>(grad_output);
+    T *gi = static_cast<T *>(grad_input);
+    OutT *gs = static_cast<OutT *>(grad_scores);
+    const int vector = vectorised ? Vec16<T>::N : 1;
+    const int64_t chunks = (args.num_columns + static_cast<int64_t>(vector) * threads - 1) /
+                           (static_cast<int64_t>(vector) * threads);
+#define FM_LAUNCH_GS(VEC, CHUNKS) \
+    grad_score_kernel<T, OutT, VEC, kFused, CHUNKS><<<rows, threads, 0, stream>>>(in, go, gi, gs, args)
+    if (vectorised) {
+        if (chunks <= 1) FM_LAUNCH_GS(true, 1);
+        else if (chunks <= 2) FM_LAUNCH_GS(true, 2);
+        else if (chunks <= 4) FM_LAUNCH_GS(true, 4);
+        else FM_LAUNCH_GS(true, 0);
+    } else {
+        FM_LAUNCH_GS(false, 0);
+    }
+#undef FM_LAUNCH_GS
+}
+
+template <bool kFused>
+static int grad_score_entry(const char *name, const void *input, const void *grad_output, const void *scores,
+                            const void *sparse_rows, void *grad_input, void *grad_scores, int64_t num_rows_dense,
+                            int64_t num_columns, int64_t num_experts_per_token, int64_t num_rows_sparse, int dtype,
+                            int scores_dtype, int out_dtype, int index_dtype, void *stream_) {
+    if (int status = validate_copy(name, input, grad_output, sparse_rows, num_rows_dense, num_columns,
+                                   num_experts_per_token, num_rows_sparse, dtype, scores_dtype, index_dtype))
+        return status;
+    FM_REQUIRE(valid_dtype(out_dtype), "%s: bad out_dtype %d", name, out_dtype);
+    if (num_rows_dense == 0 || num_experts_per_token == 0) return FM_OK;
+    FM_REQUIRE(grad_scores, "%s: null grad_scores", name);
+    if (kFused) FM_REQUIRE(scores && (grad_input || num_columns == 0), "%s: null scores or grad_input", name);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    CopyArgs args{sparse_rows, scores, num_columns, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype};
+    const int vector = 16 / dtype_size(dtype);
+    const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(grad_output) &&
+                            (!kFused || aligned16(grad_input));
+    const int threads = copy_threads(num_columns, vectorised ? vector : 1);
+    FM_DISPATCH_DTYPE(dtype, T, {
+        FM_DISPATCH_DTYPE(out_dtype, OutT, {
+            launch_grad_score<T, OutT, kFused>(input, grad_output, grad_input, grad_scores, num_rows_dense, args,
+                                               vectorised, threads, stream);
+        });
+    });
+    return check_launch(name);
+}
+
+}  // namespace fm
+
+extern "C" int fm_copy_sparse_to_dense_grad_score(const void *input, const void *grad_output, const void *sparse_rows,
+                                                  void *grad_scores, int64_t num_rows_dense, int64_t num_columns,
+                                                  int64_t num_experts_per_token, int64_t num_rows_sparse, int dtype,
+                                                  int out_dtype, int index_dtype, void *stream) {
+    return grad_score_entry<false>("fm_copy_sparse_to_dense_grad_score", input, grad_output, nullptr, sparse_rows,
+                                   nullptr, grad_scores, num_rows_dense, num_columns, num_experts_per_token,
+                                   num_rows_sparse, dtype, FM_DTYPE_F32, out_dtype, index_dtype, stream);
+}
+
+extern "C" int fm_copy_sparse_to_dense_backward(const void *input, const void *grad_output, const void *scores,
+                                                const void *sparse_rows, void *grad_input, void *grad_scores,
+                                                int64_t num_rows_dense, int64_t num_columns,
+                                                int64_t num_experts_per_token, int64_t num_rows_sparse, int dtype,
+                                                int scores_dtype, int out_dtype, int index_dtype, void *stream) {
+    return grad_score_entry<true>("fm_copy_sparse_to_dense_backward", input, grad_output, scores, sparse_rows,
+                                  grad_input, grad_scores, num_rows_dense, num_columns, num_experts_per_token,
+                                  num_rows_sparse, dtype, scores_dtype, out_dtype, index_dtype, stream);
+}

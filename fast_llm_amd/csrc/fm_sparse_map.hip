@@ -1,0 +1,198 @@
+// Routing: build the sparse map (expert histogram -> padded expert offsets -> stable row of every
+// (token, slot) pair) with integer arithmetic only, so the result is bit-exact and run-to-run identical.
+//
+// Three small launches over the flattened `top_experts` (M = tokens * experts_per_token entries):
+//   1. sparse_map_histogram_kernel: one workgroup per 1024 entries. Each wavefront finds, with
+//      ceil(log2 E) ballots, the set of lanes that hold the same expert ("match-any"); the lowest lane of each
+//      set adds the set size to an LDS histogram. The workgroup writes its E counts to the workspace.
+//   2. sparse_map_layout_kernel: one workgroup. Thread e turns column e of the per-workgroup counts into an
+//      exclusive prefix (in place) and gets count[e]; an LDS scan of the padded counts gives expert_ends,
+//      expert_pad_begins and the first row of every expert.
+//   3. sparse_map_rows_kernel: same partition as (1). rank inside the wavefront = popcount of the match set
+//      below the lane; rank inside the workgroup adds an LDS prefix over the 16 wavefronts; the global stable
+//      rank adds the exclusive prefix from (2). row = begin[e] + rank.
+// Ranks follow the flattened index order, i.e. the order of a stable sort by expert
+// (reference: fast_llm/functional/triton/sparse_copy.py:249-254).
+#include "fm_common.h"
+
+namespace fm {
+
+constexpr int kMapBlock = 1024;  // entries (= threads) per workgroup
+constexpr int kMapWaves = kMapBlock / 64;
+constexpr int kMapMaxExperts = 1024;
+
+__device__ __forceinline__ int log2_ceil(int value) {
+    int bits = 0;
+    while ((1 << bits) < value) ++bits;
+    return bits;
+}
+
+// Lanes of this wavefront whose (valid) expert equals this lane's. Undefined for invalid lanes.
+__device__ __forceinline__ uint64_t match_expert(int expert, bool valid, int num_bits) {
+    uint64_t same = __ballot(valid);
+    for (int bit = 0; bit < num_bits; ++bit) {
+        const bool set = (expert >> bit) & 1;
+        const uint64_t with_bit = __ballot(valid && set);
+        same &= set ? with_bit : ~with_bit;
+    }
+    return same;
+}
+
+__global__ __launch_bounds__(kMapBlock) void sparse_map_histogram_kernel(const int64_t *__restrict__ top_experts,
+                                                                         int64_t num_entries, int num_experts,
+                                                                         int32_t *__restrict__ block_counts) {
+    extern __shared__ int32_t lds_counts[];  // [num_experts]
+    for (int e = threadIdx.x; e < num_experts; e += kMapBlock) lds_counts[e] = 0;
+    __syncthreads();
+
+    const int64_t entry = static_cast<int64_t>(blockIdx.x) * kMapBlock + threadIdx.x;
+    int64_t expert64 = entry < num_entries ? top_experts[entry] : -1;
+    const bool valid = expert64 >= 0 && expert64 < num_experts;
+    const int expert = valid ? static_cast<int>(expert64) : 0;
+    const uint64_t same = match_expert(expert, valid, log2_ceil(num_experts));
+    const int lane = threadIdx.x & 63;
+    if (valid && (same & ((1ull << lane) - 1)) == 0) atomicAdd(&lds_counts[expert], __popcll(same));
+    __syncthreads();
+
+    int32_t *out = block_counts + static_cast<int64_t>(blockIdx.x) * num_experts;
+    for (int e = threadIdx.x; e < num_experts; e += kMapBlock) out[e] = lds_counts[e];
+}
+
+__global__ __launch_bounds__(kMapBlock) void sparse_map_layout_kernel(int32_t *__restrict__ block_counts,
+                                                                      int num_blocks, int num_experts,
+                                                                      int64_t pad_to_multiple, int index_dtype,
+                                                                      void *__restrict__ expert_ends,
+                                                                      void *__restrict__ expert_pad_begins,
+                                                                      int32_t *__restrict__ expert_begins) {
+    __shared__ int64_t lds_wave_totals[kMapWaves];
+    const int e = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    // Exclusive prefix over workgroups of this expert's counts, in place.
+    int64_t count = 0;
+    if (e < num_experts) {
+        int32_t running = 0;
+        for (int b = 0; b < num_blocks; ++b) {
+            int32_t *slot = block_counts + static_cast<int64_t>(b) * num_experts + e;
+            const int32_t here = *slot;
+            *slot = running;
+            running += here;
+        }
+        count = running;
+    }
+    const int64_t padded = (count + pad_to_multiple - 1) / pad_to_multiple * pad_to_multiple;
+
+    // Inclusive scan of `padded` over experts: wavefront scan, then the wavefront totals.
+    int64_t inclusive = padded;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        const int64_t other = __shfl_up(inclusive, offset, 64);
+        if (lane >= offset) inclusive += other;
+    }
+    if (lane == 63) lds_wave_totals[wave] = inclusive;
+    __syncthreads();
+    int64_t base = 0;
+    for (int w = 0; w < wave; ++w) base += lds_wave_totals[w];
+    inclusive += base;
+
+    if (e < num_experts) {
+        const int64_t begin = inclusive - padded;
+        store_index(expert_ends, index_dtype, e, inclusive);
+        store_index(expert_pad_begins, index_dtype, e, begin + count);
+        expert_begins[e] = static_cast<int32_t>(begin);
+    }
+}
+
+__global__ __launch_bounds__(kMapBlock) void sparse_map_rows_kernel(const int64_t *__restrict__ top_experts,
+                                                                    int64_t num_entries, int num_experts,
+                                                                    const int32_t *__restrict__ block_prefix,
+                                                                    const int32_t *__restrict__ expert_begins,
+                                                                    int index_dtype, void *__restrict__ sparse_rows) {
+    extern __shared__ int32_t lds_wave_counts[];  // [kMapWaves][num_experts]
+    for (int i = threadIdx.x; i < kMapWaves * num_experts; i += kMapBlock) lds_wave_counts[i] = 0;
+    __syncthreads();
+
+    const int64_t entry = static_cast<int64_t>(blockIdx.x) * kMapBlock + threadIdx.x;
+    int64_t expert64 = entry < num_entries ? top_experts[entry] : -1;
+    const bool valid = expert64 >= 0 && expert64 < num_experts;
+    const int expert = valid ? static_cast<int>(expert64) : 0;
+    const uint64_t same = match_expert(expert, valid, log2_ceil(num_experts));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rank_in_wave = __popcll(same & ((1ull << lane) - 1));
+    if (valid && rank_in_wave == 0) lds_wave_counts[wave * num_experts + expert] = __popcll(same);
+    __syncthreads();
+
+    // Exclusive prefix over the wavefronts of the workgroup, per expert, in place.
+    for (int e = threadIdx.x; e < num_experts; e += kMapBlock) {
+        int32_t running = 0;
+#pragma unroll
+        for (int w = 0; w < kMapWaves; ++w) {
+            const int32_t here = lds_wave_counts[w * num_experts + e];
+            lds_wave_counts[w * num_experts + e] = running;
+            running += here;
+        }
+    }
+    __syncthreads();
+
+    if (entry < num_entries) {
+        int64_t row = -1;
+        if (valid) {
+            row = static_cast<int64_t>(expert_begins[expert]) +
+                  block_prefix[static_cast<int64_t>(blockIdx.x) * num_experts + expert] +
+                  lds_wave_counts[wave * num_experts + expert] + rank_in_wave;
+        }
+        store_index(sparse_rows, index_dtype, entry, row);
+    }
+}
+
+static inline int64_t map_num_blocks(int64_t num_entries) { return (num_entries + kMapBlock - 1) / kMapBlock; }
+
+}  // namespace fm
+
+extern "C" size_t fm_sparse_map_workspace_size(int64_t num_rows_dense, int64_t num_experts_per_token,
+                                               int64_t num_experts) {
+    if (num_rows_dense < 0 || num_experts_per_token < 0 || num_experts < 0) return 0;
+    const int64_t blocks = fm::map_num_blocks(num_rows_dense * num_experts_per_token);
+    const size_t bytes = static_cast<size_t>((blocks + 1) * num_experts) * sizeof(int32_t);
+    return (bytes + 255) / 256 * 256 + 256;
+}
+
+extern "C" int fm_sparse_map(const int64_t *top_experts, int64_t num_rows_dense, int64_t num_experts_per_token,
+                             int64_t num_experts, int64_t pad_to_multiple, int index_dtype, void *sparse_rows,
+                             void *expert_ends, void *expert_pad_begins, void *workspace, size_t workspace_size,
+                             void *stream_) {
+    using namespace fm;
+    FM_REQUIRE(num_rows_dense >= 0 && num_experts_per_token >= 0, "fm_sparse_map: negative shape");
+    FM_REQUIRE(num_experts >= 1 && num_experts <= kMapMaxExperts,
+               "fm_sparse_map: num_experts=%lld outside [1, %d]", (long long)num_experts, kMapMaxExperts);
+    FM_REQUIRE(pad_to_multiple >= 1, "fm_sparse_map: pad_to_multiple=%lld < 1", (long long)pad_to_multiple);
+    FM_REQUIRE(valid_index_dtype(index_dtype), "fm_sparse_map: bad index_dtype %d", index_dtype);
+    const int64_t num_entries = num_rows_dense * num_experts_per_token;
+    const int64_t max_rows = num_entries + num_experts * pad_to_multiple;
+    FM_REQUIRE(max_rows < (int64_t(1) << 31), "fm_sparse_map: %lld padded rows overflow int32", (long long)max_rows);
+    FM_REQUIRE(index_dtype != FM_INDEX_I16 || max_rows <= 32767 + pad_to_multiple,
+               "fm_sparse_map: %lld padded rows do not fit int16", (long long)max_rows);
+    FM_REQUIRE(expert_ends && expert_pad_begins && workspace, "fm_sparse_map: null output or workspace");
+    FM_REQUIRE(num_entries == 0 || (top_experts && sparse_rows), "fm_sparse_map: null top_experts/sparse_rows");
+    FM_REQUIRE(workspace_size >= fm_sparse_map_workspace_size(num_rows_dense, num_experts_per_token, num_experts),
+               "fm_sparse_map: workspace of %zu bytes is too small", workspace_size);
+    FM_REQUIRE(aligned16(workspace), "fm_sparse_map: workspace must be 16-byte aligned");
+
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int blocks = static_cast<int>(map_num_blocks(num_entries));
+    const int experts = static_cast<int>(num_experts);
+    int32_t *block_counts = static_cast<int32_t *>(workspace);
+    int32_t *expert_begins = block_counts + static_cast<int64_t>(blocks) * experts;
+
+    if (blocks > 0) {
+        sparse_map_histogram_kernel<<<blocks, kMapBlock, experts * sizeof(int32_t), stream>>>(
+            top_experts, num_entries, experts, block_counts);
+    }
+    sparse_map_layout_kernel<<<1, kMapBlock, 0, stream>>>(block_counts, blocks, experts, pad_to_multiple, index_dtype,
+                                                          expert_ends, expert_pad_begins, expert_begins);
+    if (blocks > 0) {
+        sparse_map_rows_kernel<<<blocks, kMapBlock, kMapWaves * experts * sizeof(int32_t), stream>>>(
+            top_experts, num_entries, experts, block_counts, expert_begins, index_dtype, sparse_rows);
+    }
+    return check_launch("fm_sparse_map");
+}

@@ -1,0 +1,84 @@
+"""
+Constants and enums of the MoE hot path (reference: fast_llm/functional/config.py:8-60,106).
+"""
+
+import enum
+import typing
+
+if typing.TYPE_CHECKING:
+    import torch
+
+
+class KernelConfig:
+    """
+    Counterpart of the reference's `TritonConfig` switch (fast_llm/functional/config.py:8-28). The reference chooses
+    between Triton kernels and a torch path; here the HIP kernels are the only path, so the switch can only confirm
+    that or refuse.
+    """
+
+    POINTWISE_BLOCK_SIZE = 1024
+
+    @classmethod
+    def enabled(cls, device: "torch.device|None" = None, default: bool | None = None) -> bool:
+        if default is False:
+            raise NotImplementedError(
+                "use_triton=False asks for the reference's torch path; this package only has the HIP kernel path"
+            )
+        if device is not None and device.type != "cuda":
+            raise RuntimeError(f"the HIP kernels need a GPU tensor, got device `{device}`")
+        return True
+
+
+# The reference's name for the switch, kept so call sites read the same.
+TritonConfig = KernelConfig
+
+
+class MLPRecomputeLevel(str, enum.Enum):
+    none = "none"
+    activation = "activation"
+    activation_and_input = "activation_and_input"
+    full = "full"
+
+    def __str__(self) -> str:
+        return self.value
+
+    @property
+    def recompute_layer_1(self) -> bool:
+        return self == MLPRecomputeLevel.full
+
+    @property
+    def recompute_activation(self) -> bool:
+        return self != MLPRecomputeLevel.none
+
+    @property
+    def recompute_sparse_input(self) -> bool:
+        return self in (MLPRecomputeLevel.full, MLPRecomputeLevel.activation_and_input)
+
+
+class ActivationType(str, enum.Enum):
+    gelu = "gelu"
+    silu = "silu"
+    relu = "relu"
+    sigmoid = "sigmoid"
+    squared_relu = "squared_relu"
+    identity = "identity"
+
+    def __str__(self) -> str:
+        return self.value
+
+    @property
+    def activation_fn(self) -> typing.Callable[["torch.Tensor"], "torch.Tensor"]:
+        import torch
+
+        return {
+            ActivationType.gelu: lambda x: torch.nn.functional.gelu(x, approximate="tanh"),
+            ActivationType.silu: torch.nn.functional.silu,
+            ActivationType.relu: torch.nn.functional.relu,
+            ActivationType.sigmoid: torch.nn.functional.sigmoid,
+            ActivationType.squared_relu: lambda x: torch.pow(torch.nn.functional.relu(x), 2),
+            ActivationType.identity: lambda x: x,
+        }[self]
+
+
+# Expert blocks of the sparse layout are padded to this many rows; the grouped GEMMs rely on it.
+MAX_DROPLESS_BLOCK_SIZE_ROW = 128

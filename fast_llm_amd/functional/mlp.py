@@ -1,0 +1,365 @@
+"""
+The MoE MLP: gated activation kernels and the forward/backward orchestration with activation recomputation.
+
+Same names, positional signatures and recompute semantics as fast_llm/functional/triton/mlp.py, single GPU
+(`group` must be None, `sequence_parallel` False). Weight gradients are side effects into `weight.grad_buffer`.
+"""
+
+import typing
+
+import torch
+
+from fast_llm_amd import _lib
+from fast_llm_amd.functional.config import ActivationType, KernelConfig, MLPRecomputeLevel
+from fast_llm_amd.functional.linear import (
+    input_parallel_linear_forward,
+    maybe_transpose,
+    output_parallel_linear_backward,
+    output_parallel_linear_forward,
+    update_linear_gradients,
+)
+from fast_llm_amd.functional.sparse_copy import (
+    SparseMap,
+    copy_dense_to_sparse_backward,
+    copy_dense_to_sparse_forward,
+    copy_sparse_to_dense_backward,
+    copy_sparse_to_dense_forward,
+)
+from fast_llm_amd.functional.sparse_linear import output_sparse_matmul
+from fast_llm_amd.functional.utils import wrap_forward_backward
+
+
+def _activation_tag(activation_type: ActivationType | str) -> int:
+    name = str(activation_type.value if isinstance(activation_type, ActivationType) else activation_type)
+    if name not in _lib.ACTIVATIONS:
+        # Same set as the reference's kernels (fast_llm/functional/triton/mlp.py:49-67 has no sigmoid either).
+        raise NotImplementedError(f"activation `{name}` has no kernel")
+    return _lib.ACTIVATIONS[name]
+
+
+def mlp_activation_forward(input_: torch.Tensor, gated: bool, activation_type: ActivationType):
+    """
+    out = act(input_[..., :n]) * input_[..., n:] if gated else act(input_).
+    Reference: `triton_mlp_activation_forward`, fast_llm/functional/triton/mlp.py:142-162.
+    """
+    assert input_.is_contiguous()
+    device = _lib.require_device(input_)
+    n_cols = input_.size(-1) // (2 if gated else 1)
+    output = input_.new_empty(input_.shape[:-1] + (n_cols,))
+    with torch.cuda.device(device):
+        _lib.check(
+            _lib.lib().fm_mlp_activation_forward(
+                _lib.ptr(input_.detach()),
+                _lib.ptr(output),
+                output.numel() // n_cols if n_cols else 0,
+                n_cols,
+                int(gated),
+                _activation_tag(activation_type),
+                _lib.dtype_tag(input_.dtype),
+                _lib.stream_ptr(device),
+            )
+        )
+    return output, (input_, gated, activation_type)
+
+
+def mlp_activation_backward(grad_output: torch.Tensor, context: tuple, recompute: bool = False):
+    """
+    Input gradient of the activation, optionally with the recomputed forward output.
+    Reference: `triton_mlp_activation_backward`, fast_llm/functional/triton/mlp.py:165-190.
+    """
+    assert grad_output.is_contiguous()
+    input_, gated, activation_type = context
+    device = _lib.require_device(input_, grad_output)
+    grad_input = torch.empty_like(input_)
+    output = torch.empty_like(grad_output) if recompute else None
+    n_cols = grad_output.size(-1)
+    with torch.cuda.device(device):
+        _lib.check(
+            _lib.lib().fm_mlp_activation_backward(
+                _lib.ptr(grad_output),
+                _lib.ptr(grad_input),
+                _lib.ptr(input_.detach()),
+                _lib.ptr(output),
+                grad_output.numel() // n_cols if n_cols else 0,
+                n_cols,
+                int(gated),
+                _activation_tag(activation_type),
+                _lib.dtype_tag(input_.dtype),
+                _lib.stream_ptr(device),
+            )
+        )
+    return grad_input, output
+
+
+mlp_activation_autograd = wrap_forward_backward(mlp_activation_forward, mlp_activation_backward)
+
+# The reference's names for the same three functions.
+triton_mlp_activation_forward = mlp_activation_forward
+triton_mlp_activation_backward = mlp_activation_backward
+triton_mlp_activation_autograd = mlp_activation_autograd
+
+
+def torch_mlp_activation(input_: torch.Tensor, gated: bool, activation_type: ActivationType) -> torch.Tensor:
+    """Plain torch statement of the activation (reference: fast_llm/functional/triton/mlp.py:195-204)."""
+    if gated:
+        x1, x2 = input_.chunk(2, dim=-1)
+        return activation_type.activation_fn(x1) * x2
+    return activation_type.activation_fn(input_)
+
+
+def mlp_forward(
+    input_: torch.Tensor,
+    scores: torch.Tensor | None,
+    weight_1: torch.Tensor,
+    bias_1: torch.Tensor | None,
+    weight_2: torch.Tensor,
+    bias_2: torch.Tensor | None,
+    gated: bool,
+    activation_type: ActivationType,
+    group: typing.Any,
+    sequence_parallel: bool,
+    training: bool = True,
+    recompute_level: MLPRecomputeLevel = MLPRecomputeLevel.none,
+    transposed_layer_2_weight: bool = False,
+    sparse_map: SparseMap | None = None,
+    use_triton: bool | None = None,
+) -> tuple[torch.Tensor, list[typing.Any] | None]:
+    """
+    dispatch -> layer 1 -> activation -> layer 2 -> combine. Returns the output and the context list for
+    `mlp_backward`; `recompute_level` decides which intermediates the context keeps.
+    Reference: fast_llm/functional/triton/mlp.py:207-311.
+    """
+    if group is not None or sequence_parallel:
+        raise NotImplementedError("tensor/sequence parallelism is not part of this single-GPU path")
+    KernelConfig.enabled(input_.device, use_triton)
+
+    # Sparse copy
+    input_shape = input_.shape
+    intermediate_0 = input_ if sparse_map is None else copy_dense_to_sparse_forward(input_, sparse_map)[0]
+
+    # Layer 1
+    intermediate_1, _ = output_parallel_linear_forward(
+        intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
+    )
+
+    if recompute_level.recompute_sparse_input:
+        intermediate_0 = None
+    else:
+        input_ = None
+
+    # Activation
+    intermediate_2, _ = mlp_activation_forward(intermediate_1, gated, activation_type)
+    if recompute_level.recompute_layer_1:
+        intermediate_1 = None
+
+    # Layer 2
+    intermediate_3, _ = input_parallel_linear_forward(
+        intermediate_2, weight_2, bias_2, group, False, transposed_layer_2_weight, True, sparse_map
+    )
+
+    # Context
+    if recompute_level.recompute_activation or not training:
+        intermediate_2 = None
+
+    # Sparse copy
+    if sparse_map is None:
+        output = intermediate_3
+        intermediate_3 = None
+    else:
+        output, _ = copy_sparse_to_dense_forward(intermediate_3, scores, sparse_map)
+
+    context = (
+        [
+            input_,
+            scores,
+            intermediate_0,
+            intermediate_1,
+            intermediate_2,
+            intermediate_3,
+            weight_1,
+            bias_1,
+            weight_2,
+            bias_2,
+            gated,
+            activation_type,
+            group,
+            sequence_parallel,
+            transposed_layer_2_weight,
+            sparse_map,
+            input_shape,
+            use_triton,
+        ]
+        if training
+        else None
+    )
+    return output, context
+
+
+def mlp_backward(grad_output: torch.Tensor, context: list[typing.Any]) -> tuple[torch.Tensor, torch.Tensor]:
+    """
+    Backward of `mlp_forward`: returns (grad_input, grad_scores); weight gradients go to the grad buffers.
+    Reference: fast_llm/functional/triton/mlp.py:314-415.
+    """
+    (
+        input_,
+        scores,
+        intermediate_0,
+        intermediate_1,
+        intermediate_2,
+        intermediate_3,
+        weight_1,
+        bias_1,
+        weight_2,
+        bias_2,
+        gated,
+        activation_type,
+        group,
+        sequence_parallel,
+        transposed_layer_2_weight,
+        sparse_map,
+        input_shape,
+        use_triton,
+    ) = context
+    context.clear()
+
+    # Sparse copy
+    if sparse_map is None:
+        grad_scores = None
+    else:
+        grad_output, grad_scores = copy_sparse_to_dense_backward(grad_output, (sparse_map, intermediate_3, scores))
+
+    # Layer 2 input grad
+    weight_2_t = maybe_transpose(weight_2, transposed_layer_2_weight)
+    if sparse_map is None:
+        grad_intermediate_2 = grad_output.matmul(weight_2_t)
+    else:
+        grad_intermediate_2 = output_sparse_matmul(grad_output, weight_2_t, sparse_map)
+
+    # Sparse input recomputation
+    if intermediate_0 is None:
+        intermediate_0 = input_ if sparse_map is None else copy_dense_to_sparse_forward(input_, sparse_map)[0]
+
+    # Layer 1 recomputation
+    if intermediate_1 is None:
+        intermediate_1 = output_parallel_linear_forward(
+            intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
+        )[0]
+
+    # Activation recomputation and/or backward
+    grad_intermediate_1, intermediate_2_ = mlp_activation_backward(
+        grad_intermediate_2.contiguous(), (intermediate_1, gated, activation_type), intermediate_2 is None
+    )
+
+    # Layer 2 parameter grad
+    del grad_intermediate_2, intermediate_1
+    update_linear_gradients(
+        intermediate_2_ if intermediate_2 is None else intermediate_2,
+        weight_2,
+        bias_2,
+        grad_output,
+        transposed_layer_2_weight,
+        sparse_map,
+    )
+    del grad_output, intermediate_2, intermediate_2_
+
+    # Layer 1 backward
+    grad_input = output_parallel_linear_backward(
+        grad_intermediate_1,
+        (intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map),
+    )
+
+    # Sparse copy
+    if sparse_map is not None:
+        grad_input = copy_dense_to_sparse_backward(grad_input, (sparse_map, input_shape))
+
+    return grad_input, grad_scores
+
+
+mlp_autograd = wrap_forward_backward(mlp_forward, mlp_backward)
+
+
+def mlp_autograd_looped(
+    hidden_states: torch.Tensor,
+    scores: torch.Tensor,
+    top_experts: torch.Tensor,
+    weight_1: torch.Tensor,
+    weight_2: torch.Tensor,
+    num_experts: int,
+    gated: bool,
+    activation_type: ActivationType,
+    group: typing.Any,
+    sequence_parallel: bool,
+    training: bool = True,
+    recompute_level: MLPRecomputeLevel = MLPRecomputeLevel.none,
+) -> torch.Tensor:
+    """
+    The looped MoE: one dense MLP per expert over the tokens routed to it, output scaled by the score and added.
+    Weight gradients land in the per-expert slices of the grad buffers. On the GPU this is the slow, simple
+    alternative to the dropless path and is what the dropless path is compared with.
+    Reference: fast_llm/functional/triton/mlp.py:421-527 (the chunk bookkeeping of `ChunkWeight`/`ChunkWeightPost` is
+    done here by handing each expert a view of the weight with a view of the grad buffer).
+    """
+    from fast_llm_amd.tensor import param_get_and_unset_is_zero
+
+    scores = scores.to(hidden_states.dtype)
+    expert_mask = torch.nn.functional.one_hot(top_experts, num_classes=num_experts).permute(2, 1, 0)
+    output = torch.zeros_like(hidden_states)
+
+    is_zero = [weight.param_grad_is_zero for weight in (weight_1, weight_2)]
+    chunks = []
+    for weight, zero in zip((weight_1, weight_2), is_zero):
+        weight_chunks = weight.detach().chunk(num_experts)
+        for weight_chunk, grad_chunk in zip(weight_chunks, weight.grad_buffer.chunk(num_experts)):
+            weight_chunk.requires_grad_(weight.requires_grad)
+            weight_chunk.grad_buffer = grad_chunk
+            weight_chunk.param_grad_is_zero = zero
+        chunks.append(weight_chunks)
+
+    class _Finish(torch.autograd.Function):
+        # Runs first in backward: nothing to do. Exists so `_Start.backward` runs after every expert's backward.
+        @staticmethod
+        def forward(ctx, x):
+            return x.view_as(x)
+
+        @staticmethod
+        def backward(ctx, grad):
+            return grad
+
+    class _Start(torch.autograd.Function):
+        # Runs last in backward: experts without tokens still owe a zero gradient; consume the weight flags.
+        @staticmethod
+        def forward(ctx, x):
+            return x.view_as(x)
+
+        @staticmethod
+        def backward(ctx, grad):
+            for weight, weight_chunks in zip((weight_1, weight_2), chunks):
+                if param_get_and_unset_is_zero(weight):
+                    for weight_chunk in weight_chunks:
+                        if weight_chunk.param_grad_is_zero:
+                            weight_chunk.grad_buffer.zero_()
+            return grad
+
+    hidden_states = _Start.apply(hidden_states)
+    for expert_idx, (weight_1_chunk, weight_2_chunk) in enumerate(zip(*chunks)):
+        row, column = torch.where(expert_mask[expert_idx])
+        if column.size(0) > 0:
+            output[column] += (
+                mlp_autograd(
+                    hidden_states[column],
+                    None,
+                    weight_1_chunk,
+                    None,
+                    weight_2_chunk,
+                    None,
+                    gated,
+                    activation_type,
+                    group,
+                    sequence_parallel,
+                    training,
+                    recompute_level,
+                    True,
+                )
+                * scores[column, row, None]
+            )
+    return _Finish.apply(output)

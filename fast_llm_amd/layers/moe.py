@@ -1,0 +1,97 @@
+"""
+A single-GPU dropless mixture-of-experts MLP block built on the HIP kernel path.
+
+Covers what `MixtureOfExpertMLP` does between the router input and the block output for top-k routing
+(reference: fast_llm/layers/decoder/mlp/mixture_of_experts.py:130-213, 237-262): router logits, top-k experts, fp32
+softmax over the selected logits, sparse map, dropless MLP. Weight layout as in the reference: `layer_1.weight`
+[experts * 2 * ffn, hidden] with each expert's block ordered [gate; up] (layers/decoder/mlp/mlp.py:81-87),
+`layer_2.weight` [experts * ffn, hidden] (stored transposed, :70-79).
+"""
+
+import torch
+
+from fast_llm_amd.functional.config import ActivationType, MLPRecomputeLevel
+from fast_llm_amd.functional.mlp import mlp_autograd
+from fast_llm_amd.functional.sparse_copy import get_sparse_map
+
+
+def attach_grad_buffer(weight: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+    """Give a weight the `grad_buffer` / `param_grad_is_zero` pair the hot path writes its gradient through
+    (in the reference the training engine does this: fast_llm/engine/multi_stage/fsdp.py:258-260, 364-372)."""
+    weight.grad_buffer = torch.empty_like(weight, dtype=dtype or weight.dtype)
+    weight.param_grad_is_zero = True
+    return weight
+
+
+def topk_routing(logits: torch.Tensor, experts_per_token: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Reference: mixture_of_experts.py:243-244."""
+    top_logits, top_experts = torch.topk(logits, k=experts_per_token, dim=-1)
+    return torch.softmax(top_logits, dim=-1, dtype=torch.float32), top_experts
+
+
+class DroplessMoEMLP(torch.nn.Module):
+    def __init__(
+        self,
+        hidden_size: int,
+        intermediate_size: int,
+        experts: int,
+        experts_per_token: int,
+        *,
+        gated: bool = True,
+        activation: ActivationType = ActivationType.silu,
+        recompute_level: MLPRecomputeLevel = MLPRecomputeLevel.none,
+        dropless_dynamic_shape: bool = False,
+        full_precision_gradients: bool = False,
+        init_std: float = 0.02,
+        dtype: torch.dtype = torch.bfloat16,
+        device: torch.device | str = "cuda",
+    ):
+        super().__init__()
+        self.experts, self.experts_per_token = experts, experts_per_token
+        self.gated, self.activation = gated, activation
+        self.recompute_level, self.dropless_dynamic_shape = recompute_level, dropless_dynamic_shape
+        layer_1_rows = experts * intermediate_size * (2 if gated else 1)
+        self.router = torch.nn.Parameter(torch.empty(experts, hidden_size, dtype=dtype, device=device))
+        self.layer_1 = torch.nn.Parameter(torch.empty(layer_1_rows, hidden_size, dtype=dtype, device=device))
+        self.layer_2 = torch.nn.Parameter(
+            torch.empty(experts * intermediate_size, hidden_size, dtype=dtype, device=device)
+        )
+        with torch.no_grad():
+            for parameter in (self.router, self.layer_1, self.layer_2):
+                parameter.normal_(0, init_std)
+        grad_dtype = torch.float32 if full_precision_gradients else None
+        attach_grad_buffer(self.layer_1, grad_dtype)
+        attach_grad_buffer(self.layer_2, grad_dtype)
+
+    def route(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        logits = torch.nn.functional.linear(hidden_states, self.router)
+        return topk_routing(logits, self.experts_per_token)
+
+    def forward(
+        self,
+        input_: torch.Tensor,
+        scores: torch.Tensor | None = None,
+        top_experts: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """`scores`/`top_experts` may be passed to bypass the router (tests pin the routing that way)."""
+        hidden_states = input_.flatten(0, -2)
+        if top_experts is None:
+            scores, top_experts = self.route(hidden_states)
+        sparse_map = get_sparse_map(top_experts, self.experts, dynamic_shape=self.dropless_dynamic_shape)
+        output = mlp_autograd(
+            hidden_states,
+            scores,
+            self.layer_1,
+            None,
+            self.layer_2,
+            None,
+            gated=self.gated,
+            activation_type=self.activation,
+            group=None,
+            sequence_parallel=False,
+            training=self.training,
+            recompute_level=self.recompute_level,
+            transposed_layer_2_weight=True,
+            sparse_map=sparse_map,
+        )
+        return output.view_as(input_)

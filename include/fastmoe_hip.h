@@ -1,0 +1,191 @@
+/*
+ * fastmoe_hip.h — C ABI of the MI355X (gfx950) dropless-MoE kernel library `libfastmoe_hip.so`.
+ *
+ * Every entry point
+ *   - takes plain device pointers, 64-bit sizes/strides (in elements) and small integer enums;
+ *   - launches asynchronously on the HIP stream passed last (`void *` holding a `hipStream_t`, NULL = default
+ *     stream) and never synchronises, allocates or frees device memory, or keeps a pointer after it returns;
+ *   - returns `FM_OK` (0) or a negative `fm_status`; the message for the calling thread is read with
+ *     `fm_last_error()`. No C++ exception crosses this boundary.
+ *
+ * The reference (ServiceNow/Fast-LLM) has no FFI for this path: its "operator API" is a set of Python
+ * callables that launch Triton kernels. Each function below replaces the kernel launch inside one of those
+ * callables; the citation names the reference launch site it stands in for.
+ */
+#ifndef FASTMOE_HIP_H
+#define FASTMOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FM_VERSION 1
+
+/* Element type of activations, weights and outputs. */
+enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
+
+/* Integer type of `sparse_rows`, `expert_ends` and `expert_pad_begins`.
+ * The reference picks int16 when the padded row count is below 32768, else int32
+ * (fast_llm/functional/triton/sparse_copy.py:270); hand-built maps in its tests are int64
+ * (tests/functional/test_sparse_matmul.py:51-62). */
+enum fm_index_dtype { FM_INDEX_I16 = 0, FM_INDEX_I32 = 1, FM_INDEX_I64 = 2 };
+
+enum fm_status {
+    FM_OK = 0,
+    FM_ERR_INVALID_ARGUMENT = -1, /* bad enum, negative size, null pointer, misaligned/unsupported stride */
+    FM_ERR_UNSUPPORTED = -2,      /* valid request that this build has no kernel for */
+    FM_ERR_LAUNCH = -3            /* the HIP runtime rejected the launch */
+};
+
+/* Activation of the MLP (fast_llm/functional/config.py:50-60; the kernels implement the five the
+ * reference's Triton kernels implement, fast_llm/functional/triton/mlp.py:49-67). */
+enum fm_activation {
+    FM_ACT_GELU = 0, /* tanh approximation */
+    FM_ACT_SILU = 1,
+    FM_ACT_RELU = 2,
+    FM_ACT_SQUARED_RELU = 3,
+    FM_ACT_IDENTITY = 4
+};
+
+/* Library / ABI version (== FM_VERSION of the header it was built from). */
+int fm_version(void);
+
+/* Message of the last failing call on this thread ("" if none). The pointer stays valid until the next
+ * failing call on the same thread. */
+const char *fm_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Routing: sparse map.
+ * Replaces `sparse_histogram_kernel` + `_compute_expert_layout`
+ * (fast_llm/functional/triton/sparse_copy.py:200-221, 241-255, launched from `get_sparse_map`, :272-288).
+ *
+ *   count[e]             = #{i : top_experts.flat[i] == e}
+ *   padded[e]            = ceil(count[e] / pad_to_multiple) * pad_to_multiple
+ *   expert_ends[e]       = sum_{e' <= e} padded[e']
+ *   expert_pad_begins[e] = expert_ends[e] - padded[e] + count[e]
+ *   sparse_rows.flat[i]  = expert_ends[e] - padded[e] + #{i' < i : top_experts.flat[i'] == e},  e = top_experts.flat[i]
+ *
+ * Integer only and deterministic: the result is bit-identical from run to run. Entries of `top_experts`
+ * outside [0, num_experts) are not counted and get sparse row -1 (the copy kernels skip negative rows).
+ *
+ * `workspace` is caller-provided device scratch of at least `fm_sparse_map_workspace_size(...)` bytes,
+ * 16-byte aligned; its content on entry is irrelevant and it may be reused as soon as the stream has
+ * passed the call.
+ * --------------------------------------------------------------------------------------------------------- */
+size_t fm_sparse_map_workspace_size(int64_t num_rows_dense, int64_t num_experts_per_token, int64_t num_experts);
+
+int fm_sparse_map(const int64_t *top_experts,   /* [num_rows_dense, num_experts_per_token], contiguous */
+                  int64_t num_rows_dense, int64_t num_experts_per_token, int64_t num_experts,
+                  int64_t pad_to_multiple,
+                  int index_dtype,              /* fm_index_dtype of the three outputs */
+                  void *sparse_rows,            /* [num_rows_dense, num_experts_per_token] */
+                  void *expert_ends,            /* [num_experts] */
+                  void *expert_pad_begins,      /* [num_experts] */
+                  void *workspace, size_t workspace_size, void *stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Sparse copies. `scores` may be NULL (un-scored copy); otherwise [num_rows_dense, num_experts_per_token]
+ * of `scores_dtype`. All row-major contiguous with `num_columns` columns. `num_rows_sparse` is the row
+ * count of the sparse buffer and is only used to bound-check nothing on the device; it documents the shape.
+ * --------------------------------------------------------------------------------------------------------- */
+
+/* Dispatch: output[sparse_rows[t, j], :] = input[t, :] * (scores[t, j] or 1), product in fp32, one rounding.
+ * Rows of `output` that no (t, j) maps to are left untouched.
+ * Replaces `copy_dense_to_sparse_kernel` (sparse_copy.py:27-49, launched at :57-65). */
+int fm_copy_dense_to_sparse(const void *input, const void *scores, const void *sparse_rows, void *output,
+                            int64_t num_rows_dense, int64_t num_columns, int64_t num_experts_per_token,
+                            int64_t num_rows_sparse, int dtype, int scores_dtype, int index_dtype, void *stream);
+
+/* Combine: output[t, :] = sum_{j = 0..k-1, in that order} input[sparse_rows[t, j], :] * (scores[t, j] or 1),
+ * accumulated in fp32, one rounding.
+ * Replaces `copy_sparse_to_dense_kernel` (sparse_copy.py:69-90, launched at :97-107). */
+int fm_copy_sparse_to_dense(const void *input, const void *scores, const void *sparse_rows, void *output,
+                            int64_t num_rows_dense, int64_t num_columns, int64_t num_experts_per_token,
+                            int64_t num_rows_sparse, int dtype, int scores_dtype, int index_dtype, void *stream);
+
+/* Score gradient of the combine: grad_scores[t, j] = <input[sparse_rows[t, j], :], grad_output[t, :]> in fp32,
+ * stored as `out_dtype`.
+ * Replaces `copy_sparse_to_dense_grad_score_kernel` (sparse_copy.py:111-148, launched at :156-164). */
+int fm_copy_sparse_to_dense_grad_score(const void *input, const void *grad_output, const void *sparse_rows,
+                                       void *grad_scores, int64_t num_rows_dense, int64_t num_columns,
+                                       int64_t num_experts_per_token, int64_t num_rows_sparse, int dtype,
+                                       int out_dtype, int index_dtype, void *stream);
+
+/* Whole backward of the combine in one pass over `grad_output`:
+ *   grad_input[sparse_rows[t, j], :] = grad_output[t, :] * scores[t, j]
+ *   grad_scores[t, j]                = <input[sparse_rows[t, j], :], grad_output[t, :]>
+ * Same results as the two calls above; replaces the pair launched by `copy_sparse_to_dense_backward`
+ * (sparse_copy.py:190-194). `scores` must not be NULL. */
+int fm_copy_sparse_to_dense_backward(const void *input, const void *grad_output, const void *scores,
+                                     const void *sparse_rows, void *grad_input, void *grad_scores,
+                                     int64_t num_rows_dense, int64_t num_columns, int64_t num_experts_per_token,
+                                     int64_t num_rows_sparse, int dtype, int scores_dtype, int out_dtype,
+                                     int index_dtype, void *stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * MLP activation. `input` is [num_rows, num_columns * (gated ? 2 : 1)], `output`/`grad_output` are
+ * [num_rows, num_columns]; all contiguous. Gated: out = act(in[:, :n]) * in[:, n:]. Math in fp32.
+ * --------------------------------------------------------------------------------------------------------- */
+
+/* Replaces `triton_mlp_activation_forward_kernel` (fast_llm/functional/triton/mlp.py:29-71, launched :153-162). */
+int fm_mlp_activation_forward(const void *input, void *output, int64_t num_rows, int64_t num_columns, int gated,
+                              int activation, int dtype, void *stream);
+
+/* grad_input has the shape of input. `output` (may be NULL) receives the recomputed forward output.
+ * Replaces `triton_mlp_activation_backward_kernel` (mlp.py:74-139, launched :177-189). */
+int fm_mlp_activation_backward(const void *grad_output, void *grad_input, const void *input, void *output,
+                               int64_t num_rows, int64_t num_columns, int gated, int activation, int dtype,
+                               void *stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Grouped ("sparse") matrix products. Strides are in elements. `lhs`/`rhs` share `dtype`; `out` has
+ * `out_dtype`; accumulation is fp32 with a single rounding at the store. With `accumulate` != 0 the previous
+ * content of `out` is added (in fp32) before the store. `expert_ends` (and `expert_pad_begins`) have
+ * `index_dtype`; the expert of a 128-row block is `#{e : expert_ends[e] <= first row of the block}`, so every
+ * expert boundary must be a multiple of 128 rows (the reference's MAX_DROPLESS_BLOCK_SIZE_ROW contract,
+ * fast_llm/functional/config.py:106, sparse_linear.py:274). If `expert_ends` is NULL the product is an
+ * ordinary dense one (a single expert owning all rows), which is what the reference does for
+ * `sparse_map=None` (sparse_linear.py:276-277, 404-405, 537-538).
+ * Results are deterministic (no split-K, no floating-point atomics).
+ * --------------------------------------------------------------------------------------------------------- */
+
+/* out[i, j] = sum_k lhs[i, k] * rhs[k, j + col_sparse_dim * e(i)]   for i < expert_ends[-1]; rows past the last
+ * expert ("phantom" rows) are neither read nor written. Padding rows inside an expert are computed like
+ * real rows. lhs [row_dim, inner_dim], rhs [inner_dim, col_sparse_dim * num_experts], out [row_dim, col_sparse_dim].
+ * Replaces `output_sparse_matmul_kernel` (sparse_linear.py:185-258, launched :288-306). */
+int fm_output_sparse_matmul(const void *lhs, const void *rhs, void *out, const void *expert_ends,
+                            int64_t row_dim, int64_t col_sparse_dim, int64_t inner_dim, int64_t num_experts,
+                            int64_t lhs_stride_row, int64_t lhs_stride_inner, int64_t rhs_stride_inner,
+                            int64_t rhs_stride_col, int64_t out_stride_row, int64_t out_stride_col,
+                            int accumulate, int dtype, int out_dtype, int index_dtype, void *stream);
+
+/* out[i, j] = sum_k lhs[i, k] * rhs[k + inner_sparse_dim * e(i), j]; same row rules as above.
+ * lhs [row_dim, inner_sparse_dim], rhs [inner_sparse_dim * num_experts, col_dim], out [row_dim, col_dim].
+ * Replaces `input_inner_sparse_matmul_kernel` (sparse_linear.py:310-385, launched :415-433). */
+int fm_input_inner_sparse_matmul(const void *lhs, const void *rhs, void *out, const void *expert_ends,
+                                 int64_t row_dim, int64_t col_dim, int64_t inner_sparse_dim, int64_t num_experts,
+                                 int64_t lhs_stride_row, int64_t lhs_stride_inner, int64_t rhs_stride_inner,
+                                 int64_t rhs_stride_col, int64_t out_stride_row, int64_t out_stride_col,
+                                 int accumulate, int dtype, int out_dtype, int index_dtype, void *stream);
+
+/* out[i + row_sparse_dim * e, j] = sum_{k in [begin_e, expert_pad_begins[e])} lhs[i, k] * rhs[k, j],
+ * begin_e = expert_ends[e - 1] (0 for e = 0). Rows of the inner dimension outside that range (padding and
+ * phantom rows) are replaced by zero before the multiply, so NaN/Inf stored there cannot leak. An expert
+ * without rows gives zeros (or leaves `out` unchanged when accumulating).
+ * lhs [row_sparse_dim, inner_dim], rhs [inner_dim, col_dim], out [row_sparse_dim * num_experts, col_dim].
+ * Replaces `input_row_sparse_matmul_kernel` (sparse_linear.py:437-517, launched :551-569). */
+int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void *out, const void *expert_ends,
+                               const void *expert_pad_begins, int64_t row_sparse_dim, int64_t col_dim,
+                               int64_t inner_dim, int64_t num_experts, int64_t lhs_stride_row,
+                               int64_t lhs_stride_inner, int64_t rhs_stride_inner, int64_t rhs_stride_col,
+                               int64_t out_stride_row, int64_t out_stride_col, int accumulate, int dtype,
+                               int out_dtype, int index_dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FASTMOE_HIP_H */

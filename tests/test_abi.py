@@ -1,0 +1,92 @@
+"""The C-ABI boundary without a GPU: the library loads, exports every symbol the header declares, and the host side
+rejects bad calls with the reference's exception types before any kernel is launched."""
+
+import ctypes
+import pathlib
+import re
+
+import pytest
+import torch
+
+from fast_llm_amd import _lib
+from fast_llm_amd.functional import sparse_copy, sparse_linear
+from fast_llm_amd.functional.config import ActivationType, KernelConfig, MLPRecomputeLevel
+from fast_llm_amd.functional.utils import div
+
+HEADER = pathlib.Path(__file__).resolve().parent.parent / "include" / "fastmoe_hip.h"
+
+
+def _declared_symbols() -> dict[str, int]:
+    """name -> number of parameters, parsed from the header."""
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    symbols = {}
+    for match in re.finditer(r"\b(?:int|size_t|const char \*)\s*(fm_\w+)\s*\(([^)]*)\)\s*;", text):
+        params = match.group(2).strip()
+        symbols[match.group(1)] = 0 if params in ("", "void") else params.count(",") + 1
+    return symbols
+
+
+def test_header_symbols_are_bound_and_exported(library):
+    declared = _declared_symbols()
+    assert len(declared) >= 13
+    assert set(declared) == set(_lib.SIGNATURES)
+    raw = ctypes.CDLL(str(_lib.LIBRARY_PATH))
+    for name, num_params in declared.items():
+        assert hasattr(raw, name), f"{name} not exported"
+        assert len(_lib.SIGNATURES[name][1]) == num_params, name
+    assert library.fm_version() == _lib.FM_VERSION
+    assert library.fm_last_error() == b""
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(_lib.FastMoeLibraryError, match="only compute path"):
+        _lib.load_library(tmp_path / "libfastmoe_hip.so")
+
+
+def test_workspace_size_is_host_only(library):
+    assert library.fm_sparse_map_workspace_size(8192, 2, 8) >= (16 + 1) * 8 * 4
+    assert library.fm_sparse_map_workspace_size(0, 2, 8) > 0
+    assert library.fm_sparse_map_workspace_size(-1, 2, 8) == 0
+
+
+def test_argument_validation_returns_status_and_message(library):
+    # Validation happens before any HIP call, so it can be exercised without a device.
+    status = library.fm_sparse_map(None, 4, 2, 0, 128, 1, None, None, None, None, 0, None)
+    assert status == _lib.FM_ERR_INVALID_ARGUMENT
+    assert b"num_experts" in library.fm_last_error()
+    with pytest.raises(ValueError, match="num_experts"):
+        _lib.check(status)
+    status = library.fm_mlp_activation_forward(None, None, 4, 4, 1, 99, 1, None)
+    assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"activation" in library.fm_last_error()
+    status = library.fm_output_sparse_matmul(None, None, None, None, 128, 128, 64, 1, 64, 1, 1, 64, 128, 1, 0, 7, 0, 1, None)
+    assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"dtype" in library.fm_last_error()
+
+
+def test_cpu_tensors_are_refused_not_emulated(library):
+    top_experts = torch.zeros(4, 2, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="GPU"):
+        sparse_copy.get_sparse_map(top_experts, 8)
+    with pytest.raises(NotImplementedError):
+        sparse_copy.get_sparse_map(top_experts, 8, use_triton=False)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        sparse_linear.dense_matmul(torch.zeros(4, 4), torch.zeros(4, 4))
+
+
+def test_shape_errors_follow_the_reference_conventions():
+    sparse_map = sparse_copy.SparseMap(None, torch.tensor([128, 256]), torch.tensor([100, 200]), None, 256, None, 3, None)
+    with pytest.raises(AssertionError):  # row_dim != num_rows
+        sparse_linear.output_sparse_matmul(torch.zeros(128, 8), torch.zeros(8, 6), sparse_map)
+    with pytest.raises(ValueError):  # columns not divisible by the expert count
+        sparse_linear.output_sparse_matmul(torch.zeros(256, 8), torch.zeros(8, 8), sparse_map)
+    with pytest.raises(AssertionError):  # accumulate without out
+        sparse_linear.input_row_sparse_matmul(torch.zeros(8, 256), torch.zeros(256, 8), sparse_map, accumulate=True)
+    with pytest.raises(ValueError):
+        div(7, 2)
+
+
+def test_enums_mirror_the_reference():
+    assert [level.value for level in MLPRecomputeLevel] == ["none", "activation", "activation_and_input", "full"]
+    assert MLPRecomputeLevel.full.recompute_layer_1 and not MLPRecomputeLevel.activation.recompute_sparse_input
+    assert MLPRecomputeLevel("activation_and_input").recompute_sparse_input
+    assert ActivationType.silu.value == "silu" and f"{ActivationType.gelu}" == "gelu"
+    assert KernelConfig.POINTWISE_BLOCK_SIZE == 1024

@@ -1,0 +1,211 @@
+"""The composed dropless MoE MLP on the GPU: the reference's `test_dropless_mlp`, the benchmark configurations
+against the oracle, and the gradient-buffer contract."""
+
+import pytest
+import torch
+
+from fast_llm_amd.functional.config import ActivationType, MLPRecomputeLevel
+from fast_llm_amd.functional.mlp import mlp_autograd, mlp_autograd_looped
+from fast_llm_amd.functional.sparse_copy import get_sparse_map
+from fast_llm_amd.layers.moe import DroplessMoEMLP, attach_grad_buffer
+from fast_llm_amd.workloads import WORKLOADS, MoEWorkload, make_inputs
+from oracle import moe_oracle
+from tests.helpers import REFERENCE_FIXTURES, max_rel_err, rms_diff
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_dropless(inputs, workload, device, recompute_level=MLPRecomputeLevel.none, grad_dtype=None, repeat=1):
+    x = inputs.hidden_states.to(device).requires_grad_(True)
+    scores = inputs.scores.to(device).requires_grad_(True)
+    weight_1 = inputs.weight_1.to(device).requires_grad_(True)
+    weight_2 = inputs.weight_2.to(device).requires_grad_(True)
+    for weight in (weight_1, weight_2):
+        attach_grad_buffer(weight, grad_dtype)
+    sparse_map = get_sparse_map(inputs.top_experts.to(device), workload.experts)
+    for _ in range(repeat):
+        output = mlp_autograd(
+            x, scores, weight_1, None, weight_2, None, True, ActivationType.silu, None, False, True,
+            recompute_level, True, sparse_map,
+        )
+        output.backward(inputs.grad_output.to(device))
+    return output.detach(), x.grad, scores.grad, weight_1.grad_buffer, weight_2.grad_buffer
+
+
+_NAMES = ("output", "grad_input", "grad_scores", "grad_weight_1", "grad_weight_2")
+
+
+def test_dropless_mlp_like_the_reference(device):
+    """tests/functional/test_functional.py:89-183: dropless vs looped within the reference's rms thresholds, and
+    bit-equal results for all four recompute levels."""
+    fixture = REFERENCE_FIXTURES["dropless_mlp"]
+    experts, top_k, std = fixture["experts"], fixture["experts_per_token"], fixture["std"]
+    tokens, hidden, ffn = fixture["tokens"], fixture["hidden"], fixture["ffn"]
+    torch.manual_seed(0)
+    input_ = torch.randn(tokens, hidden, device=device, requires_grad=True)
+    router_weight = torch.normal(0, std, (experts, hidden), device=device)
+    top_logits, top_experts = torch.topk(torch.nn.functional.linear(input_.detach(), router_weight), k=top_k, dim=-1)
+    scores = torch.softmax(top_logits, dim=-1, dtype=torch.float32).detach().requires_grad_()
+    output_grad = torch.randn(tokens, hidden, device=device)
+    weight_1 = torch.normal(0, std, (ffn * 2 * experts, hidden), device=device, requires_grad=True)
+    weight_2 = torch.normal(0, std, (ffn * experts, hidden), device=device, requires_grad=True)
+    params = (weight_1, weight_2)
+
+    for param in params:
+        attach_grad_buffer(param)
+    output_ref = mlp_autograd_looped(
+        input_, scores, top_experts, weight_1, weight_2, experts, True, ActivationType.silu, None, False, True,
+        MLPRecomputeLevel.none,
+    )
+    output_ref.backward(output_grad)
+    input_grad_ref, scores_grad_ref = input_.grad, scores.grad
+    param_grad_refs = [param.grad_buffer for param in params]
+    assert not any(param.param_grad_is_zero for param in params)
+
+    sparse_map = get_sparse_map(top_experts, experts)
+    for i, recompute_level in enumerate(MLPRecomputeLevel):
+        input_.grad = None
+        scores.grad = None
+        for param in params:
+            param.grad = None
+            attach_grad_buffer(param)
+        output = mlp_autograd(
+            input_, scores, weight_1, None, weight_2, None, True, ActivationType.silu, None, False, True,
+            recompute_level, True, sparse_map,
+        )
+        output.backward(output_grad)
+        assert all(param.grad is None for param in params)  # weight gradients only through the buffers
+        if i == 0:
+            assert rms_diff(output, output_ref) <= fixture["rms_output"]
+            assert rms_diff(input_.grad, input_grad_ref) <= fixture["rms_input_grad"]
+            assert rms_diff(scores.grad, scores_grad_ref) <= fixture["rms_scores_grad"]
+            for param, param_grad_ref in zip(params, param_grad_refs):
+                assert rms_diff(param.grad_buffer, param_grad_ref) <= fixture["rms_weight_grad"]
+            # fp32 here, so the tighter benchmark bound holds as well
+            assert max_rel_err(output, output_ref) <= 1e-5
+            assert max_rel_err(input_.grad, input_grad_ref) <= 1e-5
+            output_ref, input_grad_ref, scores_grad_ref = output, input_.grad, scores.grad
+            param_grad_refs = [param.grad_buffer for param in params]
+        else:
+            # Recomputation doesn't modify the output.
+            assert torch.equal(output, output_ref), recompute_level
+            assert torch.equal(input_.grad, input_grad_ref), recompute_level
+            assert torch.equal(scores.grad, scores_grad_ref), recompute_level
+            for param, param_grad_ref in zip(params, param_grad_refs):
+                assert torch.equal(param.grad_buffer, param_grad_ref), recompute_level
+
+
+def test_tiny_configuration_fp32_against_cpu_oracle(device):
+    """Benchmark configuration 1 (512 tokens, hidden 256, ffn 512, 8 experts, top-2, fp32): every output and gradient
+    within max relative error 1e-5 of the CPU looped MoE and of the CPU dropless restatement."""
+    workload = WORKLOADS["tiny"]
+    inputs = make_inputs(workload, seed=0)
+    actual = _run_dropless(inputs, workload, device)
+    looped = moe_oracle.looped_moe_forward_backward(
+        inputs.hidden_states, inputs.scores, inputs.top_experts, inputs.weight_1, inputs.weight_2, workload.experts,
+        inputs.grad_output,
+    )
+    dropless = moe_oracle.dropless_mlp_forward_backward(
+        inputs.hidden_states, inputs.scores, inputs.weight_1, inputs.weight_2,
+        moe_oracle.sparse_map(inputs.top_experts, workload.experts), inputs.grad_output,
+    )
+    for name, ours in zip(_NAMES, actual):
+        assert max_rel_err(ours.cpu(), getattr(looped, name)) <= 1e-5, name
+        assert max_rel_err(ours.cpu(), getattr(dropless, name)) <= 1e-5, name
+
+
+@pytest.mark.parametrize(
+    "workload",
+    [
+        MoEWorkload("small_bf16", 1024, 512, 768, 8, 2, torch.bfloat16),
+        MoEWorkload("small_bf16_many_experts", 2048, 256, 384, 64, 6, torch.bfloat16),
+        MoEWorkload("small_bf16_empty", 512, 512, 256, 8, 2, torch.bfloat16, zipf_exponent=1.2, empty_experts=(1, 6)),
+        MoEWorkload("small_fp16", 512, 256, 512, 4, 2, torch.float16),
+    ],
+    ids=lambda workload: workload.name,
+)
+def test_small_half_precision_against_cpu_oracle(workload, device):
+    """bf16/fp16 storage with fp32 accumulation: max relative error 1e-2 against the oracle evaluated with the same
+    storage roundings, and against the fp32 looped MoE on the same (half-precision) inputs."""
+    inputs = make_inputs(workload, seed=3)
+    actual = _run_dropless(inputs, workload, device)
+    sparse_map = moe_oracle.sparse_map(inputs.top_experts, workload.experts)
+    dropless = moe_oracle.dropless_mlp_forward_backward(
+        inputs.hidden_states, inputs.scores, inputs.weight_1, inputs.weight_2, sparse_map, inputs.grad_output
+    )
+    looped = moe_oracle.looped_moe_forward_backward(
+        inputs.hidden_states.float(), inputs.scores, inputs.top_experts, inputs.weight_1.float(),
+        inputs.weight_2.float(), workload.experts, inputs.grad_output.float(),
+    )
+    for name, ours in zip(_NAMES, actual):
+        assert torch.isfinite(ours).all(), name
+        assert max_rel_err(ours.cpu(), getattr(dropless, name)) <= 1e-2, name
+        # The fp32 looped path never rounds intermediates to bf16: allow for those roundings too.
+        assert max_rel_err(ours.cpu(), getattr(looped, name)) <= 2e-2, name
+    if workload.empty_experts:
+        ffn = workload.ffn
+        for expert in workload.empty_experts:
+            assert (actual[4][expert * ffn : (expert + 1) * ffn] == 0).all()
+            assert (actual[3][expert * 2 * ffn : (expert + 1) * 2 * ffn] == 0).all()
+
+
+def test_grad_buffer_contract(device):
+    """First backward overwrites the (uninitialised) buffer and clears `param_grad_is_zero`; the next accumulates;
+    fp32 buffers under bf16 compute are honoured (fast_llm/functional/linear.py:47-55, fast_llm/tensor.py:345-348)."""
+    workload = MoEWorkload("contract", 512, 256, 256, 4, 2, torch.bfloat16)
+    inputs = make_inputs(workload, seed=4)
+    once = _run_dropless(inputs, workload, device, grad_dtype=torch.float32)
+    twice = _run_dropless(inputs, workload, device, grad_dtype=torch.float32, repeat=2)
+    assert once[3].dtype == torch.float32
+    for single, double in zip(once[3:], twice[3:]):
+        assert max_rel_err(double, 2 * single) <= 1e-6
+    bf16_buffers = _run_dropless(inputs, workload, device)
+    for single, low in zip(once[3:], bf16_buffers[3:]):
+        assert low.dtype == torch.bfloat16
+        assert max_rel_err(low, single) <= 1e-2
+
+
+def test_moe_module_routes_and_runs(device):
+    torch.manual_seed(0)
+    layer = DroplessMoEMLP(256, 384, 8, 2, dtype=torch.bfloat16, device=device, recompute_level=MLPRecomputeLevel.activation)
+    x = torch.randn(4, 96, 256, device=device, dtype=torch.bfloat16, requires_grad=True)
+    out = layer(x)
+    out.backward(torch.randn_like(out))
+    assert out.shape == x.shape and torch.isfinite(out).all() and torch.isfinite(x.grad).all()
+    assert not layer.layer_1.param_grad_is_zero and torch.isfinite(layer.layer_1.grad_buffer).all()
+    scores, top_experts = layer.route(x.detach().flatten(0, 1))
+    looped = moe_oracle.looped_moe(
+        x.detach().flatten(0, 1).float(), scores, top_experts, layer.layer_1.detach().float(),
+        layer.layer_2.detach().float(), 8,
+    )
+    assert max_rel_err(out.detach().flatten(0, 1), looped) <= 2e-2
+    layer.eval()
+    with torch.no_grad():
+        assert torch.equal(layer(x), out)
+
+
+@pytest.mark.parametrize("name", ["mixtral", "fine_grained", "wide", "imbalanced", "imbalanced_empty"])
+def test_benchmark_configurations_full_size(name, device):
+    """Configurations 2-5 at full size. The CPU oracle would need minutes per case, so the checker is the oracle's
+    looped MoE evaluated by torch on the GPU in fp32 (per-expert dense matmuls + autograd) on the same inputs."""
+    if name == "imbalanced_empty":
+        workload = MoEWorkload(name, 8192, 4096, 14336, 8, 2, torch.bfloat16, zipf_exponent=1.2, empty_experts=(5,))
+    else:
+        workload = WORKLOADS[name]
+    inputs = make_inputs(workload, seed=7)
+    actual = _run_dropless(inputs, workload, device)
+    torch.cuda.synchronize()
+    gpu = inputs.to(device)
+    expected = moe_oracle.looped_moe_forward_backward(
+        gpu.hidden_states.float(), gpu.scores, gpu.top_experts, gpu.weight_1.float(), gpu.weight_2.float(),
+        workload.experts, gpu.grad_output.float(),
+    )
+    for name_, ours in zip(_NAMES, actual):
+        assert torch.isfinite(ours).all(), name_
+        error = max_rel_err(ours, getattr(expected, name_))
+        assert error <= 1e-2, f"{name_}: {error}"
+    counts = torch.bincount(inputs.top_experts.flatten(), minlength=workload.experts)
+    if name.startswith("imbalanced"):
+        assert counts.max() > 2.5 * counts.float().mean()
+    if workload.empty_experts:
+        assert counts[5] == 0 and (actual[4][5 * workload.ffn : 6 * workload.ffn] == 0).all()

@@ -1,0 +1,238 @@
+"""The three grouped matrix products on the GPU: the reference's own fixtures and tolerances
+(tests/functional/test_sparse_matmul.py), then layouts, dtypes, accumulation, padding and phantom rows."""
+
+import pytest
+import torch
+
+from fast_llm_amd.functional.sparse_linear import (
+    InputSparseLinear,
+    OutputSparseLinear,
+    dense_matmul,
+    input_inner_sparse_matmul,
+    input_row_sparse_matmul,
+    output_sparse_matmul,
+)
+from oracle import moe_oracle
+from tests.helpers import REFERENCE_FIXTURES, fixture_sparse_map, max_rel_err, rms_diff, to_device_map
+
+pytestmark = pytest.mark.gpu
+
+_CASES = REFERENCE_FIXTURES["sparse_matmul"]["cases"]
+_STD = REFERENCE_FIXTURES["sparse_matmul"]["std"]
+_RMS = REFERENCE_FIXTURES["sparse_matmul"]["rms_tolerance"]
+# max|a - b| / max|b| per tensor: fp32 multiply-add vs bf16/fp16 operands with fp32 accumulation.
+_MAX_REL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 2e-3}
+
+
+def _normal(rows, columns, dtype, generator):
+    return torch.normal(0, _STD, (rows, columns), generator=generator).to(dtype)
+
+
+def _used_rows(oracle_map):
+    return int(oracle_map.expert_ends[-1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", _CASES)
+@pytest.mark.parametrize("index_dtype", [torch.int64, torch.int16])
+def test_output_sparse_matmul(case, dtype, index_dtype, device):
+    generator = torch.Generator().manual_seed(0)
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device, index_dtype)
+    lhs = _normal(oracle_map.num_rows, case["dense_dim"], dtype, generator)
+    rhs = _normal(case["dense_dim"], case["sparse_dim"] * oracle_map.num_experts, dtype, generator)
+    # Randomly initialize the output to ensure padded values have no effect.
+    out = _normal(oracle_map.num_rows, case["sparse_dim"], dtype, generator).to(device)
+    output = output_sparse_matmul(lhs.to(device), rhs.to(device), sparse_map, out)
+    assert output is out
+    expected = moe_oracle.output_sparse_matmul(lhs, rhs, oracle_map)
+    assert rms_diff(output.cpu(), expected) <= _RMS
+    assert max_rel_err(output.cpu(), expected) <= _MAX_REL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", _CASES)
+def test_input_inner_sparse_matmul(case, dtype, device):
+    generator = torch.Generator().manual_seed(1)
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device)
+    lhs = _normal(oracle_map.num_rows, case["sparse_dim"], dtype, generator)
+    rhs = _normal(case["sparse_dim"] * oracle_map.num_experts, case["dense_dim"], dtype, generator)
+    output = input_inner_sparse_matmul(lhs.to(device), rhs.to(device), sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(lhs, rhs, oracle_map)
+    assert rms_diff(output.cpu(), expected) <= _RMS
+    assert max_rel_err(output.cpu(), expected) <= _MAX_REL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", _CASES)
+def test_input_row_sparse_matmul(case, dtype, device):
+    generator = torch.Generator().manual_seed(2)
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device)
+    lhs = _normal(case["sparse_dim"], oracle_map.num_rows, dtype, generator)
+    rhs = _normal(oracle_map.num_rows, case["dense_dim"], dtype, generator)
+    output = input_row_sparse_matmul(lhs.to(device), rhs.to(device), sparse_map)
+    expected = moe_oracle.input_row_sparse_matmul(lhs, rhs, oracle_map)
+    assert rms_diff(output.cpu(), expected) <= _RMS
+    assert max_rel_err(output.cpu(), expected) <= _MAX_REL[dtype]
+    if 0 in case["tokens_per_expert"]:
+        empty = case["tokens_per_expert"].index(0)
+        assert (output[empty * case["sparse_dim"] : (empty + 1) * case["sparse_dim"]] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", _CASES)
+@pytest.mark.parametrize(
+    ("autograd_class", "expert_axis"), [(OutputSparseLinear, 1), (InputSparseLinear, 0)], ids=["output", "input"]
+)
+def test_sparse_linear_autograd(case, dtype, autograd_class, expert_axis, device):
+    """Mirror of the reference's `test_sparse_linear_autograd` (test_sparse_matmul.py:198-233): per-expert reference
+    on the real rows, padded rows of out and grad_lhs zeroed before comparing."""
+    generator = torch.Generator().manual_seed(3)
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device)
+    experts, tokens = oracle_map.num_experts, oracle_map.num_rows
+    if expert_axis == 1:
+        lhs_features, out_features = case["dense_dim"], case["sparse_dim"]
+        rhs_shape = (case["dense_dim"], case["sparse_dim"] * experts)
+    else:
+        lhs_features, out_features = case["sparse_dim"], case["dense_dim"]
+        rhs_shape = (case["sparse_dim"] * experts, case["dense_dim"])
+    lhs = _normal(tokens, lhs_features, dtype, generator)
+    rhs = _normal(*rhs_shape, dtype, generator)
+    grad_output = _normal(tokens, out_features, dtype, generator)
+
+    lhs_ref = lhs.float().requires_grad_(True)
+    rhs_ref = rhs.float().requires_grad_(True)
+    out_ref = lhs_ref.new_zeros(tokens, out_features)
+    begins = oracle_map.expert_begins.tolist()
+    pad_begins = oracle_map.expert_pad_begins.tolist()
+    for i, rhs_chunk in enumerate(rhs_ref.chunk(experts, dim=expert_axis)):
+        out_ref[begins[i] : pad_begins[i]] = lhs_ref[begins[i] : pad_begins[i]] @ rhs_chunk
+    out_ref.backward(grad_output.float())
+
+    lhs_t = lhs.to(device).requires_grad_(True)
+    rhs_t = rhs.to(device).requires_grad_(True)
+    out_t = autograd_class.apply(lhs_t, rhs_t, sparse_map)
+    out_t.backward(grad_output.to(device))
+
+    def zero_padded(tensor):
+        masked = tensor.detach().cpu().float().clone()
+        masked[~oracle_map.real_row_mask()] = 0
+        return masked
+
+    tolerance = _MAX_REL[dtype]
+    assert rms_diff(zero_padded(out_t), out_ref.detach()) <= _RMS
+    assert rms_diff(zero_padded(lhs_t.grad), lhs_ref.grad) <= _RMS
+    assert rms_diff(rhs_t.grad.cpu().float(), rhs_ref.grad) <= _RMS
+    assert max_rel_err(zero_padded(out_t), out_ref.detach()) <= tolerance
+    assert max_rel_err(zero_padded(lhs_t.grad), lhs_ref.grad) <= tolerance
+    assert max_rel_err(rhs_t.grad.cpu().float(), rhs_ref.grad) <= tolerance
+
+
+def _moe_layout(dtype, generator, rows_per_expert=(256, 0, 128, 384), tokens=(200, 0, 128, 300), phantom=256,
+                hidden=256, ffn=384):
+    """The operand layouts of the MoE layer (weights [E*N, H], transposed views) with an empty expert, a full one,
+    ragged ones and a phantom tail."""
+    ends, total = [], 0
+    for rows in rows_per_expert:
+        total += rows
+        ends.append(total)
+    case = {"expert_ends": ends, "tokens_per_expert": list(tokens)}
+    oracle_map = fixture_sparse_map(case)
+    oracle_map.num_rows = total + phantom
+    experts = len(ends)
+    x = _normal(oracle_map.num_rows, hidden, dtype, generator)
+    y = _normal(oracle_map.num_rows, ffn, dtype, generator)
+    weight = _normal(experts * ffn, hidden, dtype, generator)
+    return oracle_map, x, y, weight
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_moe_layer_layouts_padding_and_phantom_rows(dtype, device):
+    generator = torch.Generator().manual_seed(4)
+    oracle_map, x, y, weight = _moe_layout(dtype, generator)
+    sparse_map = to_device_map(oracle_map, device, torch.int16)
+    used, tolerance = _used_rows(oracle_map), _MAX_REL[dtype]
+    real = oracle_map.real_row_mask()
+    x_gpu, y_gpu, weight_gpu = x.to(device), y.to(device), weight.to(device)
+
+    # Layer-1-like: rhs = weight.t(), reduction-contiguous. Phantom rows of a pre-filled out must survive.
+    out = torch.full((oracle_map.num_rows, weight.size(0) // 4), 7.0, dtype=dtype, device=device)
+    output_sparse_matmul(x_gpu, weight_gpu.t(), sparse_map, out)
+    expected = moe_oracle.output_sparse_matmul(x, weight.t(), oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+    assert (out[used:] == 7.0).all()
+
+    # Layer-2-like: rhs = weight row-major, expert blocks along the reduction axis.
+    out = input_inner_sparse_matmul(y_gpu, weight_gpu, sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(y, weight, oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+
+    # Weight gradient: lhs = y.t() (a transposed view), NaN/Inf in every padding and phantom row of both operands.
+    y_poisoned, x_poisoned = y.clone(), x.clone()
+    y_poisoned[~real] = float("nan")
+    x_poisoned[~real] = float("inf")
+    for out_dtype in (dtype, torch.float32):
+        out = torch.full(weight.shape, 3.0, dtype=out_dtype, device=device)
+        input_row_sparse_matmul(y_poisoned.to(device).t(), x_poisoned.to(device), sparse_map, out=out)
+        expected = moe_oracle.input_row_sparse_matmul(y.t(), x, oracle_map, out=torch.zeros(weight.shape, dtype=out_dtype))
+        assert torch.isfinite(out).all()
+        assert max_rel_err(out.cpu(), expected) <= tolerance
+        ffn = weight.size(0) // 4
+        assert (out[ffn : 2 * ffn] == 0).all()  # the empty expert gets zeros, not stale memory
+        # accumulate=True adds to what is there, including for the empty expert
+        input_row_sparse_matmul(y_poisoned.to(device).t(), x_poisoned.to(device), sparse_map, out=out, accumulate=True)
+        assert max_rel_err(out.cpu(), 2 * expected.float()) <= tolerance
+        assert (out[ffn : 2 * ffn] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_accumulate_and_wider_output(dtype, device):
+    generator = torch.Generator().manual_seed(5)
+    case = _CASES[0]
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device)
+    lhs = _normal(oracle_map.num_rows, case["dense_dim"], dtype, generator)
+    rhs = _normal(case["dense_dim"], case["sparse_dim"] * 3, dtype, generator)
+    previous = _normal(oracle_map.num_rows, case["sparse_dim"], torch.float32, generator)
+    out = previous.to(device)
+    output_sparse_matmul(lhs.to(device), rhs.to(device), sparse_map, out, accumulate=True)
+    expected = moe_oracle.output_sparse_matmul(lhs, rhs, oracle_map, out=previous.clone(), accumulate=True)
+    assert out.dtype == torch.float32
+    assert max_rel_err(out.cpu(), expected) <= _MAX_REL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(("rows", "inner", "columns"), [(256, 128, 256), (384, 192, 128), (100, 70, 36), (1, 1, 1)])
+def test_dense_matmul_and_odd_shapes(rows, inner, columns, dtype, device):
+    generator = torch.Generator().manual_seed(6)
+    lhs, rhs = _normal(rows, inner, dtype, generator), _normal(inner, columns, dtype, generator)
+    expected = (lhs.float() @ rhs.float()).to(dtype)
+    assert max_rel_err(dense_matmul(lhs.to(device), rhs.to(device)).cpu(), expected) <= _MAX_REL[dtype]
+    assert max_rel_err(output_sparse_matmul(lhs.to(device), rhs.to(device), None).cpu(), expected) <= _MAX_REL[dtype]
+    # transposed operands, consumed through their strides
+    lhs_t, rhs_t = lhs.t().contiguous().to(device).t(), rhs.t().contiguous().to(device).t()
+    assert max_rel_err(dense_matmul(lhs_t, rhs_t).cpu(), expected) <= _MAX_REL[dtype]
+
+
+def test_results_are_bit_identical_from_run_to_run(device):
+    generator = torch.Generator().manual_seed(7)
+    oracle_map, x, y, weight = _moe_layout(torch.bfloat16, generator, hidden=512, ffn=512)
+    sparse_map = to_device_map(oracle_map, device, torch.int16)
+    x_gpu, y_gpu, weight_gpu = x.to(device), y.to(device), weight.to(device)
+    used = _used_rows(oracle_map)
+    first = (
+        output_sparse_matmul(x_gpu, weight_gpu.t(), sparse_map)[:used],
+        input_inner_sparse_matmul(y_gpu, weight_gpu, sparse_map)[:used],
+        input_row_sparse_matmul(y_gpu.t(), x_gpu, sparse_map),
+    )
+    for _ in range(3):
+        again = (
+            output_sparse_matmul(x_gpu, weight_gpu.t(), sparse_map)[:used],
+            input_inner_sparse_matmul(y_gpu, weight_gpu, sparse_map)[:used],
+            input_row_sparse_matmul(y_gpu.t(), x_gpu, sparse_map),
+        )
+        for a, b in zip(first, again):
+            assert torch.equal(a, b)
