@@ -1,0 +1,195 @@
+"""
+Benchmark of the dropless-MoE hot path on one MI355X.
+
+A step is one forward + backward of the MoE MLP over one batch of synthetic tokens: sparse map, dispatch, layer 1,
+gated SiLU, layer 2, combine, and the whole backward including both weight gradients. Inputs, weights and routing
+(top-k experts, fp32 scores) are resident in HBM before the timed region. The default workload is the Mixtral-like
+configuration (8192 tokens, hidden 4096, ffn 14336, 8 experts, top-2, bf16 with fp32 accumulation).
+
+Prints one JSON line: whole-step tokens/s, the roofline of the grouped-GEMM kernel (six launches per step, algorithmic
+FLOPs 18*M*H*F over their summed device time from HIP events on the launch stream), per-kernel figures for the
+bandwidth-bound kernels, and a CPU baseline (the looped torch MoE on the host cores, on a bounded token sample).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E peak, GB/s
+
+
+def parse_args() -> argparse.Namespace:
+    parser = argparse.ArgumentParser(description=__doc__)
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=10)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--workload", default="mixtral", help="tiny | mixtral | fine_grained | wide | imbalanced")
+    parser.add_argument("--recompute", default="none", help="none | activation | activation_and_input | full")
+    parser.add_argument("--cpu-tokens", type=int, default=512, help="tokens in the CPU baseline sample (0: skip)")
+    parser.add_argument("--seed", type=int, default=0)
+    return parser.parse_args()
+
+
+def cpu_baseline(workload, inputs, tokens: int) -> dict:
+    """The looped torch MoE (per-expert gather -> linear -> silu*up -> linear -> scaled scatter-add, autograd
+    backward) in fp32 on the host cores, over the first `tokens` tokens of the same batch with all experts' weights."""
+    from oracle import moe_oracle
+
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "1024")))))
+    weight_1, weight_2 = inputs.weight_1.float().cpu(), inputs.weight_2.float().cpu()
+    x, grad = inputs.hidden_states[:tokens].float().cpu(), inputs.grad_output[:tokens].float().cpu()
+    scores, top_experts = inputs.scores[:tokens].cpu(), inputs.top_experts[:tokens].cpu()
+
+    def run(count: int) -> float:
+        start = time.perf_counter()
+        moe_oracle.looped_moe_forward_backward(
+            x[:count], scores[:count], top_experts[:count], weight_1, weight_2, workload.experts, grad[:count]
+        )
+        return time.perf_counter() - start
+
+    run(min(tokens, 32))  # thread pool and allocator warm-up
+    seconds = run(tokens)
+    return {
+        "value": tokens / seconds,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"first {tokens} of {workload.tokens} tokens, full {workload.experts}-expert weights, fp32, "
+        f"looped torch MoE fwd+bwd, 1 warm-up + 1 timed pass ({seconds:.2f} s)",
+    }
+
+
+def main() -> None:
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(
+            "bench.py measures one GPU: the dropless-MoE path keeps the whole expert set on a single MI355X and has no "
+            "collectives. Run it with --gpus 1.",
+            file=sys.stderr,
+        )
+        sys.exit(2)
+
+    from fast_llm_amd import _lib
+    from fast_llm_amd.functional.config import ActivationType, MLPRecomputeLevel
+    from fast_llm_amd.functional.mlp import mlp_autograd
+    from fast_llm_amd.functional.sparse_copy import get_sparse_map
+    from fast_llm_amd.layers.moe import attach_grad_buffer
+    from fast_llm_amd.workloads import WORKLOADS, make_inputs
+
+    if not _lib.LIBRARY_PATH.is_file():
+        from fast_llm_amd.build import build_library
+
+        build_library()
+
+    workload = WORKLOADS[args.workload]
+    recompute_level = MLPRecomputeLevel(args.recompute)
+    device = torch.device("cuda:0")
+    inputs = make_inputs(workload, seed=args.seed, weight_device=device).to(device)
+    x = inputs.hidden_states.requires_grad_(True)
+    scores = inputs.scores.requires_grad_(True)
+    weight_1 = attach_grad_buffer(inputs.weight_1.requires_grad_(True))
+    weight_2 = attach_grad_buffer(inputs.weight_2.requires_grad_(True))
+
+    def step() -> None:
+        x.grad = scores.grad = None
+        weight_1.param_grad_is_zero = weight_2.param_grad_is_zero = True
+        sparse_map = get_sparse_map(inputs.top_experts, workload.experts)
+        output = mlp_autograd(
+            x, scores, weight_1, None, weight_2, None, True, ActivationType.silu, None, False, True,
+            recompute_level, True, sparse_map,
+        )
+        output.backward(inputs.grad_output)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    with _lib.KernelTimer() as timer:
+        start = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - start
+    ms_per_step = seconds / args.steps * 1e3
+    tokens_per_second = workload.tokens * args.steps / seconds
+
+    # Per-kernel device time, averaged over the timed steps.
+    durations = {label: sum(values) / len(values) for label, values in timer.durations_ms().items()}
+    calls_per_step = {label: len(values) / args.steps for label, values in timer.durations_ms().items()}
+    rows, hidden, ffn = workload.sparse_rows_unpadded, workload.hidden, workload.ffn
+    itemsize = workload.dtype.itemsize
+    gemm_ms = sum(durations[label] * calls_per_step[label] for label in durations if "matmul" in label)
+    gemm_flops = workload.gemm_flops * (4 / 3 if recompute_level.recompute_layer_1 else 1)
+    gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
+    index_size = 2 if rows + workload.experts * 128 < 32768 else 4
+    copy_bytes = workload.copy_bytes + rows * (index_size + 4)  # rows + indices + fp32 scores
+    kernels = {}
+    for label, ms in sorted(durations.items()):
+        entry = {"ms": round(ms, 4), "calls_per_step": calls_per_step[label]}
+        if "matmul" in label:
+            m, n, k = (int(v) for v in label[label.index("[") + 1 : -1].split("x"))
+            # Dimensions are padded/static; algorithmic FLOPs use the unpadded row count.
+            per_launch = 2 * rows * (n if "row_sparse" not in label else m) * (k if "row_sparse" not in label else n)
+            entry["tflops"] = round(per_launch / (ms * 1e-3) / 1e12, 1)
+            entry["frac_of_mfma_peak"] = round(entry["tflops"] / PEAK_BF16_TFLOPS, 4)
+        elif label in ("fm_copy_dense_to_sparse", "fm_copy_sparse_to_dense"):
+            entry["gbs"] = round(copy_bytes / (ms * 1e-3) / 1e9, 1)
+            entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
+        elif label == "fm_copy_sparse_to_dense_backward":
+            fused_bytes = (1 + 2 * workload.experts_per_token) * workload.tokens * hidden * itemsize
+            entry["gbs"] = round(fused_bytes / (ms * 1e-3) / 1e9, 1)
+            entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
+        elif label.startswith("fm_mlp_activation"):
+            factor = 3 if label.endswith("forward") else (6 if recompute_level.recompute_activation else 5)
+            entry["gbs"] = round(factor * rows * ffn * itemsize / (ms * 1e-3) / 1e9, 1)
+            entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
+        kernels[label] = entry
+
+    result = {
+        "metric": "MoE fwd+bwd tokens/s at Mixtral shape; grouped-GEMM % bf16 MFMA peak",
+        "value": tokens_per_second,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[workload.dtype],
+        "data": "synthetic",
+        "config": {
+            "workload": f"{workload.name}: dropless MoE MLP fwd+bwd, {workload.tokens} tokens, hidden {hidden}, "
+            f"ffn {ffn}, {workload.experts} experts, top-{workload.experts_per_token}, gated SiLU, "
+            f"recompute={recompute_level.value}",
+            "tokens": workload.tokens,
+            "hidden": hidden,
+            "ffn": ffn,
+            "experts": workload.experts,
+            "experts_per_token": workload.experts_per_token,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "grouped_gemm_mfma_kernel (six launches per step)",
+            "achieved": gemm_tflops,
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": gemm_tflops / PEAK_BF16_TFLOPS,
+            "traffic": None,
+            "flops_per_step": gemm_flops,
+            "ms_per_step": gemm_ms,
+        },
+        "gemm_frac_of_step": gemm_ms / ms_per_step,
+        "kernels": kernels,
+    }
+    if args.cpu_tokens > 0:
+        result["cpu_baseline"] = cpu_baseline(workload, inputs, min(args.cpu_tokens, workload.tokens))
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -87,6 +87,53 @@ def check(status: int) -> None:
     raise ValueError(message)
 
 
+class KernelTimer:
+    """
+    Device-time of every kernel-library call made while the timer is active, from HIP events recorded on the launch
+    stream right before and after the call. Used by the benchmark; costs two event records per call.
+    """
+
+    def __init__(self):
+        self.records: list[tuple[str, torch.cuda.Event, torch.cuda.Event]] = []
+
+    def __enter__(self) -> "KernelTimer":
+        global _active_timer
+        self._previous, _active_timer = _active_timer, self
+        return self
+
+    def __exit__(self, *exc) -> None:
+        global _active_timer
+        _active_timer = self._previous
+
+    def durations_ms(self) -> dict[str, list[float]]:
+        """label -> device milliseconds of each call, in call order. Synchronises."""
+        torch.cuda.synchronize()
+        out: dict[str, list[float]] = {}
+        for label, start, end in self.records:
+            out.setdefault(label, []).append(start.elapsed_time(end))
+        return out
+
+
+_active_timer: KernelTimer | None = None
+
+
+def call(name: str, device: torch.device, *args, label: str | None = None) -> None:
+    """Launch entry point `name` on the current stream of `device` (appended as the last argument) and raise on a
+    non-zero status."""
+    function = getattr(lib(), name)
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device)
+        timer = _active_timer
+        if timer is not None:
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(stream)
+        status = function(*args, stream.cuda_stream)
+        if timer is not None:
+            end.record(stream)
+            timer.records.append((label or name, start, end))
+    check(status)
+
+
 def require_device(*tensors: torch.Tensor | None) -> torch.device:
     """All tensors must live on one HIP device; there is no host implementation to fall back to."""
     device = None

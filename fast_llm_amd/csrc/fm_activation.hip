@@ -10,24 +10,6 @@ namespace fm {
 
 constexpr int kActThreads = 256;
 
-template <int kActivation>
-__device__ __forceinline__ float activation_forward(float x) {
-    if constexpr (kActivation == FM_ACT_GELU) {
-        const float tanh_input = 0.79788456f * x * (1.f + 0.044715f * x * x);
-        const float tanh_value = 1.f - 2.f / (1.f + expf(2.f * tanh_input));
-        return x * 0.5f * (1.f + tanh_value);
-    } else if constexpr (kActivation == FM_ACT_SILU) {
-        return x / (1.f + expf(-x));
-    } else if constexpr (kActivation == FM_ACT_RELU) {
-        return x > 0.f ? x : 0.f;
-    } else if constexpr (kActivation == FM_ACT_SQUARED_RELU) {
-        const float relu = x > 0.f ? x : 0.f;
-        return relu * relu;
-    } else {
-        return x;
-    }
-}
-
 // Returns act'(x) and writes act(x) to `out`.
 template <int kActivation>
 __device__ __forceinline__ float activation_backward(float x, float &out) {
@@ -53,6 +35,15 @@ __device__ __forceinline__ float activation_backward(float x, float &out) {
         out = x;
         return 1.f;
     }
+}
+
+// The forward value is taken from the same expression the backward kernel uses when it recomputes the output,
+// so a recomputed activation is bit-identical to the stored one.
+template <int kActivation>
+__device__ __forceinline__ float activation_forward(float x) {
+    float out;
+    (void)activation_backward<kActivation>(x, out);
+    return out;
 }
 
 template <typename T, int kActivation, bool kGated, bool kVector>

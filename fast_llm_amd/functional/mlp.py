@@ -46,19 +46,17 @@ def mlp_activation_forward(input_: torch.Tensor, gated: bool, activation_type: A
     device = _lib.require_device(input_)
     n_cols = input_.size(-1) // (2 if gated else 1)
     output = input_.new_empty(input_.shape[:-1] + (n_cols,))
-    with torch.cuda.device(device):
-        _lib.check(
-            _lib.lib().fm_mlp_activation_forward(
-                _lib.ptr(input_.detach()),
-                _lib.ptr(output),
-                output.numel() // n_cols if n_cols else 0,
-                n_cols,
-                int(gated),
-                _activation_tag(activation_type),
-                _lib.dtype_tag(input_.dtype),
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        "fm_mlp_activation_forward",
+        device,
+        _lib.ptr(input_.detach()),
+        _lib.ptr(output),
+        output.numel() // n_cols if n_cols else 0,
+        n_cols,
+        int(gated),
+        _activation_tag(activation_type),
+        _lib.dtype_tag(input_.dtype),
+    )
     return output, (input_, gated, activation_type)
 
 
@@ -73,21 +71,19 @@ def mlp_activation_backward(grad_output: torch.Tensor, context: tuple, recompute
     grad_input = torch.empty_like(input_)
     output = torch.empty_like(grad_output) if recompute else None
     n_cols = grad_output.size(-1)
-    with torch.cuda.device(device):
-        _lib.check(
-            _lib.lib().fm_mlp_activation_backward(
-                _lib.ptr(grad_output),
-                _lib.ptr(grad_input),
-                _lib.ptr(input_.detach()),
-                _lib.ptr(output),
-                grad_output.numel() // n_cols if n_cols else 0,
-                n_cols,
-                int(gated),
-                _activation_tag(activation_type),
-                _lib.dtype_tag(input_.dtype),
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        "fm_mlp_activation_backward",
+        device,
+        _lib.ptr(grad_output),
+        _lib.ptr(grad_input),
+        _lib.ptr(input_.detach()),
+        _lib.ptr(output),
+        grad_output.numel() // n_cols if n_cols else 0,
+        n_cols,
+        int(gated),
+        _activation_tag(activation_type),
+        _lib.dtype_tag(input_.dtype),
+    )
     return grad_input, output
 
 

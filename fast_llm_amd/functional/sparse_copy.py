@@ -63,23 +63,21 @@ def get_sparse_map(
     library = _lib.lib()
     workspace_size = library.fm_sparse_map_workspace_size(num_rows_dense, num_experts_per_token, num_experts)
     workspace = torch.empty(workspace_size, dtype=torch.uint8, device=device)
-    with torch.cuda.device(device):
-        _lib.check(
-            library.fm_sparse_map(
-                _lib.ptr(top_experts),
-                num_rows_dense,
-                num_experts_per_token,
-                num_experts,
-                pad_to_multiple,
-                _lib.index_tag(dtype),
-                _lib.ptr(sparse_rows),
-                _lib.ptr(expert_ends),
-                _lib.ptr(expert_pad_begins),
-                _lib.ptr(workspace),
-                workspace_size,
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        "fm_sparse_map",
+        device,
+        _lib.ptr(top_experts),
+        num_rows_dense,
+        num_experts_per_token,
+        num_experts,
+        pad_to_multiple,
+        _lib.index_tag(dtype),
+        _lib.ptr(sparse_rows),
+        _lib.ptr(expert_ends),
+        _lib.ptr(expert_pad_begins),
+        _lib.ptr(workspace),
+        workspace_size,
+    )
     return SparseMap(
         sparse_rows=sparse_rows,
         expert_ends=expert_ends,
@@ -123,20 +121,18 @@ def copy_dense_to_sparse(input_: torch.Tensor, scores: torch.Tensor | None, spar
     # A worst-case static shape.
     out = input_.new_empty((sparse_map.num_rows, input_.size(1)))
     shape = _copy_arguments(input_, out, scores, sparse_map)
-    with torch.cuda.device(device):
-        _lib.check(
-            _lib.lib().fm_copy_dense_to_sparse(
-                _lib.ptr(input_),
-                _lib.ptr(scores),
-                _lib.ptr(sparse_map.sparse_rows),
-                _lib.ptr(out),
-                *shape[:4],
-                shape[4],
-                shape[5],
-                shape[6],
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        "fm_copy_dense_to_sparse",
+        device,
+        _lib.ptr(input_),
+        _lib.ptr(scores),
+        _lib.ptr(sparse_map.sparse_rows),
+        _lib.ptr(out),
+        *shape[:4],
+        shape[4],
+        shape[5],
+        shape[6],
+    )
     return out
 
 
@@ -148,20 +144,18 @@ def copy_sparse_to_dense(input_: torch.Tensor, scores: torch.Tensor | None, spar
     device = _lib.require_device(input_, scores, sparse_map.sparse_rows)
     out = input_.new_empty((sparse_map.num_rows_dense, input_.size(1)))
     shape = _copy_arguments(out, input_, scores, sparse_map)
-    with torch.cuda.device(device):
-        _lib.check(
-            _lib.lib().fm_copy_sparse_to_dense(
-                _lib.ptr(input_),
-                _lib.ptr(scores),
-                _lib.ptr(sparse_map.sparse_rows),
-                _lib.ptr(out),
-                *shape[:4],
-                shape[4],
-                shape[5],
-                shape[6],
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        "fm_copy_sparse_to_dense",
+        device,
+        _lib.ptr(input_),
+        _lib.ptr(scores),
+        _lib.ptr(sparse_map.sparse_rows),
+        _lib.ptr(out),
+        *shape[:4],
+        shape[4],
+        shape[5],
+        shape[6],
+    )
     return out
 
 
@@ -175,20 +169,18 @@ def copy_sparse_to_dense_grad_score(
     device = _lib.require_device(input_, grad_output, sparse_map.sparse_rows)
     out = input_.new_empty(sparse_map.num_rows_dense, sparse_map.num_experts_per_token)
     shape = _copy_arguments(grad_output, input_, None, sparse_map)
-    with torch.cuda.device(device):
-        _lib.check(
-            _lib.lib().fm_copy_sparse_to_dense_grad_score(
-                _lib.ptr(input_),
-                _lib.ptr(grad_output),
-                _lib.ptr(sparse_map.sparse_rows),
-                _lib.ptr(out),
-                *shape[:4],
-                shape[4],
-                _lib.dtype_tag(out.dtype),
-                shape[6],
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        "fm_copy_sparse_to_dense_grad_score",
+        device,
+        _lib.ptr(input_),
+        _lib.ptr(grad_output),
+        _lib.ptr(sparse_map.sparse_rows),
+        _lib.ptr(out),
+        *shape[:4],
+        shape[4],
+        _lib.dtype_tag(out.dtype),
+        shape[6],
+    )
     return out
 
 
@@ -229,23 +221,21 @@ def copy_sparse_to_dense_backward(grad_output: torch.Tensor, context: tuple[Spar
     grad_scores = input_.new_empty(sparse_map.num_rows_dense, sparse_map.num_experts_per_token)
     shape = _copy_arguments(grad_output, input_, scores, sparse_map)
     Assert.eq(input_.shape, grad_input.shape)
-    with torch.cuda.device(device):
-        _lib.check(
-            _lib.lib().fm_copy_sparse_to_dense_backward(
-                _lib.ptr(input_),
-                _lib.ptr(grad_output),
-                _lib.ptr(scores),
-                _lib.ptr(sparse_map.sparse_rows),
-                _lib.ptr(grad_input),
-                _lib.ptr(grad_scores),
-                *shape[:4],
-                shape[4],
-                shape[5],
-                _lib.dtype_tag(grad_scores.dtype),
-                shape[6],
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        "fm_copy_sparse_to_dense_backward",
+        device,
+        _lib.ptr(input_),
+        _lib.ptr(grad_output),
+        _lib.ptr(scores),
+        _lib.ptr(sparse_map.sparse_rows),
+        _lib.ptr(grad_input),
+        _lib.ptr(grad_scores),
+        *shape[:4],
+        shape[4],
+        shape[5],
+        _lib.dtype_tag(grad_scores.dtype),
+        shape[6],
+    )
     return grad_input, grad_scores
 
 

@@ -42,25 +42,24 @@ def _launch(
     pointers = [_lib.ptr(lhs.detach()), _lib.ptr(rhs.detach()), _lib.ptr(out), _lib.ptr(expert_ends)]
     if with_pad_begins:
         pointers.append(_lib.ptr(expert_pad_begins))
-    with torch.cuda.device(device):
-        _lib.check(
-            getattr(_lib.lib(), name)(
-                *pointers,
-                *dims,
-                num_experts,
-                lhs.stride(0),
-                lhs.stride(1),
-                rhs.stride(0),
-                rhs.stride(1),
-                out.stride(0),
-                out.stride(1),
-                int(accumulate),
-                _lib.dtype_tag(lhs.dtype),
-                _lib.dtype_tag(out.dtype),
-                _lib.index_tag(index_dtype),
-                _lib.stream_ptr(device),
-            )
-        )
+    _lib.call(
+        name,
+        device,
+        *pointers,
+        *dims,
+        num_experts,
+        lhs.stride(0),
+        lhs.stride(1),
+        rhs.stride(0),
+        rhs.stride(1),
+        out.stride(0),
+        out.stride(1),
+        int(accumulate),
+        _lib.dtype_tag(lhs.dtype),
+        _lib.dtype_tag(out.dtype),
+        _lib.index_tag(index_dtype),
+        label=f"{name}[{dims[0]}x{dims[1]}x{dims[2]}]",
+    )
     return out
 
 

@@ -60,11 +60,17 @@ class MoEInputs:
     top_experts: torch.Tensor  # [T, k] int64
 
     def to(self, device: torch.device | str) -> "MoEInputs":
-        return MoEInputs(**{key: value.to(device) for key, value in dataclasses.asdict(self).items()})
+        return MoEInputs(**{field.name: getattr(self, field.name).to(device) for field in dataclasses.fields(self)})
 
 
-def make_inputs(workload: MoEWorkload, seed: int = 0, weights: bool = True) -> MoEInputs:
-    """x, grad ~ N(0, 1); router and expert weights ~ N(0, 0.02); top-k routing with fp32 softmax over the top logits."""
+def make_inputs(
+    workload: MoEWorkload, seed: int = 0, weights: bool = True, weight_device: torch.device | None = None
+) -> MoEInputs:
+    """
+    x, grad ~ N(0, 1); router and expert weights ~ N(0, 0.02); top-k routing with fp32 softmax over the top logits.
+    Everything is drawn on the CPU unless `weight_device` is given: then the (large) expert weights are drawn there
+    from a generator of that device, which is much faster but not bit-reproducible on another device.
+    """
     generator = torch.Generator().manual_seed(seed)
 
     def normal(shape, std):
@@ -81,7 +87,15 @@ def make_inputs(workload: MoEWorkload, seed: int = 0, weights: bool = True) -> M
         logits[:, expert] = float("-inf")
     top_logits, top_experts = torch.topk(logits, k=workload.experts_per_token, dim=-1)
     scores = torch.softmax(top_logits, dim=-1, dtype=torch.float32)
-    if weights:
+    if weights and weight_device is not None:
+        device_generator = torch.Generator(device=weight_device).manual_seed(seed)
+        weight_1, weight_2 = (
+            torch.empty((workload.experts * width, workload.hidden), dtype=workload.dtype, device=weight_device).normal_(
+                0, 0.02, generator=device_generator
+            )
+            for width in (2 * workload.ffn, workload.ffn)
+        )
+    elif weights:
         weight_1 = torch.empty((workload.experts * 2 * workload.ffn, workload.hidden), dtype=workload.dtype)
         weight_2 = torch.empty((workload.experts * workload.ffn, workload.hidden), dtype=workload.dtype)
         # Filled in slabs so the fp32 staging buffer stays small next to the 1.9 GB bf16 weight.

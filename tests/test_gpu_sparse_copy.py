@@ -55,8 +55,18 @@ def test_dispatch_and_combine(tokens, experts, top_k, hidden, dtype, scored, dev
     dispatched = copy_dense_to_sparse(dense.to(device), gpu_scores, sparse_map).cpu()
     expected = moe_oracle.copy_dense_to_sparse(dense, scores if scored else None, oracle_map)
     assert dispatched.shape == expected.shape
-    # A single fp32 product rounded once: bit-exact, scored or not.
-    assert torch.equal(dispatched[mask], expected[mask])
+    if scored and dtype == torch.float16:
+        # The fp16 product is rounded once from the exact value (fused multiply-convert), the oracle rounds it to
+        # fp32 first: results may differ by one fp16 ulp on rare ties.
+        ulp = torch.finfo(dtype).eps * expected[mask].float().abs().clamp_min(2.0**-14)
+        assert ((dispatched[mask].float() - expected[mask].float()).abs() <= ulp).all()
+    else:
+        # A copy, or a single fp32 product rounded once: bit-exact.
+        different = dispatched[mask] != expected[mask]
+        assert not different.any(), (
+            f"{different.sum().item()} of {different.numel()} differ, e.g. "
+            f"{dispatched[mask][different][:4].tolist()} vs {expected[mask][different][:4].tolist()}"
+        )
 
     combined = copy_sparse_to_dense(sparse.to(device), gpu_scores, sparse_map).cpu()
     expected = moe_oracle.copy_sparse_to_dense(sparse, scores if scored else None, oracle_map)

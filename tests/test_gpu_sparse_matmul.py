@@ -103,8 +103,8 @@ def test_sparse_linear_autograd(case, dtype, autograd_class, expert_axis, device
     rhs = _normal(*rhs_shape, dtype, generator)
     grad_output = _normal(tokens, out_features, dtype, generator)
 
-    lhs_ref = lhs.float().requires_grad_(True)
-    rhs_ref = rhs.float().requires_grad_(True)
+    lhs_ref = lhs.float().clone().requires_grad_(True)
+    rhs_ref = rhs.float().clone().requires_grad_(True)
     out_ref = lhs_ref.new_zeros(tokens, out_features)
     begins = oracle_map.expert_begins.tolist()
     pad_begins = oracle_map.expert_pad_begins.tolist()
