@@ -1,48 +1,22 @@
-// Grouped ("sparse") matrix products of the dropless MoE MLP on gfx950 matrix cores.
+// Grouped ("sparse") matrix products of the dropless MoE MLP: entry points, dispatch, and the generic kernel.
 //
-// One kernel template serves the three products; they differ only in how an output tile finds its operands:
-//   output-sparse      : 128-row block -> expert e -> columns [e*N_s, (e+1)*N_s) of rhs
-//   input-inner-sparse : 128-row block -> expert e -> rows    [e*K_s, (e+1)*K_s) of rhs
-//   input-row-sparse   : 128-row block of out -> expert e -> reduction over rows [begin_e, pad_begin_e) of the
-//                        token axis, everything outside replaced by zero when it is staged into LDS
+// The three products differ only in how an output tile finds its operands:
+//   output-sparse      : row block -> expert e -> columns [e*N_s, (e+1)*N_s) of rhs
+//   input-inner-sparse : row block -> expert e -> rows    [e*K_s, (e+1)*K_s) of rhs
+//   input-row-sparse   : row block of out -> expert e -> reduction over rows [begin_e, pad_begin_e) of the
+//                        token axis, everything outside replaced by zero before the multiply
 // (reference semantics: fast_llm/functional/triton/sparse_linear.py:185-258, 310-385, 437-517).
 //
-// Fast path (bf16/fp16): workgroup tile 128 x BN x 64, four wavefronts in a 2 x 2 grid, each wavefront owns
-// 64 x BN/2 of the tile as 32x32x16 MFMA accumulators in fp32. Operand tiles go HBM -> registers (16-byte
-// vectors, prefetched one K-step ahead) -> LDS (XOR-swizzled 16-byte chunks, conflict-free for both the
-// writes and the 128-bit fragment reads) -> MFMA. Either operand may be contiguous along the reduction axis or
-// along its other axis; both end up in the same LDS layout, so the inner loop is identical.
-// Workgroups are renumbered so that consecutive tiles run on the same XCD (shared L2) and walk a group of row
-// blocks before moving to the next column block.
-//
-// Generic path (fp32, or any shape/stride the fast path does not take): 64 x 64 x 16 LDS-tiled FMA kernel
-// with full bounds checks; fp32 multiply-add, so it also serves the 1e-5 parity configuration.
-#include "fm_common.h"
+// Half-precision operands with vectorisable layouts go to the MFMA kernel (fm_gemm_mfma.hip). Everything else
+// (fp32 operands, odd strides or sizes) goes to the generic kernel below: a 64 x 64 x 16 LDS-tiled kernel with
+// full bounds checks and true fp32 multiply-adds, which is also what the 1e-5 fp32 parity bound needs. The
+// generic kernel takes the expert of a 64-row block from its first row, so there expert boundaries must be
+// multiples of 64 rows.
+#include "fm_gemm_common.h"
 
 namespace fm {
 
-enum GemmMode { kOutputSparse = 0, kInputInnerSparse = 1, kInputRowSparse = 2 };
-
-struct GemmArgs {
-    const void *lhs;
-    const void *rhs;
-    void *out;
-    const void *expert_ends;        // null: dense product
-    const void *expert_pad_begins;  // row-sparse mode only
-    int64_t lhs_stride_row, lhs_stride_inner, rhs_stride_inner, rhs_stride_col, out_stride_row, out_stride_col;
-    int64_t rows;         // rows of out
-    int64_t cols;         // columns of out
-    int64_t inner;        // length of the reduction axis as stored (per expert for input-inner-sparse)
-    int64_t sparse_size;  // N_s, K_s or M_s
-    int num_experts;
-    int mode;
-    int accumulate;
-    int index_dtype;
-    int out_dtype;
-    int tiles_m, tiles_n;
-};
-
-// Where one output tile reads and writes. Offsets are in elements.
+// Where one output tile of the generic kernel reads and writes. Offsets are in elements.
 struct TileWork {
     int64_t lhs_offset;  // element (first row of tile, k = 0)
     int64_t rhs_offset;  // element (k = 0, first column of tile)
@@ -94,212 +68,6 @@ __device__ __forceinline__ TileWork resolve_tile(const GemmArgs &args, int64_t r
                               col0 * args.rhs_stride_col;
     }
     return work;
-}
-
-// Map the hardware workgroup id to a tile. Hardware deals consecutive ids round-robin to the 8 XCDs; undo that
-// so each XCD gets a contiguous range of logical ids, then walk `kGroupRows` row blocks per column block.
-__device__ __forceinline__ void tile_of_block(const GemmArgs &args, int &tile_m, int &tile_n) {
-    constexpr int kXcds = 8, kGroupRows = 16;
-    const int total = args.tiles_m * args.tiles_n;
-    const int pid = blockIdx.x;
-    const int per_xcd = (total + kXcds - 1) / kXcds;
-    const int tall = total % kXcds == 0 ? kXcds : total % kXcds;
-    const int xcd = pid % kXcds, local = pid / kXcds;
-    const int logical = xcd < tall ? xcd * per_xcd + local : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
-    const int width = kGroupRows * args.tiles_n;
-    const int group = logical / width;
-    const int first_m = group * kGroupRows;
-    const int group_rows = min(args.tiles_m - first_m, kGroupRows);
-    const int in_group = logical - group * width;
-    tile_m = first_m + in_group % group_rows;
-    tile_n = in_group / group_rows;
-}
-
-template <typename OutT>
-__device__ __forceinline__ void store_out(void *out, int64_t offset, float value, bool accumulate) {
-    OutT *pointer = static_cast<OutT *>(out) + offset;
-    if (accumulate) value += to_float(*pointer);
-    *pointer = from_float<OutT>(value);
-}
-
-__device__ __forceinline__ void store_out_dyn(void *out, int out_dtype, int64_t offset, float value, bool accumulate) {
-    if (out_dtype == FM_DTYPE_F32) store_out<float>(out, offset, value, accumulate);
-    else if (out_dtype == FM_DTYPE_BF16) store_out<bf16_t>(out, offset, value, accumulate);
-    else store_out<f16_t>(out, offset, value, accumulate);
-}
-
-// =========================================================================================================
-// Fast path
-// =========================================================================================================
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
-typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
-
-template <typename T>
-struct Mfma;
-template <>
-struct Mfma<bf16_t> {
-    static __device__ __forceinline__ f32x16_t run(u32x4_t a, u32x4_t b, f32x16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
-                                                       c, 0, 0, 0);
-    }
-};
-template <>
-struct Mfma<f16_t> {
-    static __device__ __forceinline__ f32x16_t run(u32x4_t a, u32x4_t b, f32x16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b),
-                                                      c, 0, 0, 0);
-    }
-};
-
-constexpr int kBM = 128, kBK = 64, kGemmThreads = 256;
-constexpr int kChunksPerRow = kBK / 8;  // 16-byte chunks along K in one LDS row
-
-// Byte offset of chunk `chunk` (8 elements along K) of row `row` in an LDS operand tile [rows][kBK].
-// The XOR spreads 16 consecutive rows of one chunk column over all 64 banks.
-__device__ __forceinline__ int lds_chunk_offset(int row, int chunk) {
-    return row * (kBK * 2) + ((chunk ^ ((row >> 1) & 7)) << 4);
-}
-
-// Stage one operand tile (kRows x kBK) from global memory into registers.
-// kContiguousK: element (r, k) at base[r * stride + k]; chunk q -> row q / 8, K-chunk q % 8.
-// otherwise   : element (r, k) at base[k * stride + r]; chunk q -> K-row q / (kRows / 8), row-chunk q % (kRows / 8).
-template <typename T, int kRows, bool kContiguousK>
-struct OperandStage {
-    static constexpr int kChunks = kRows * kChunksPerRow / kGemmThreads;
-    u32x4_t regs[kChunks];
-
-    __device__ __forceinline__ void load(const T *base, int64_t stride, int64_t k0) {
-#pragma unroll
-        for (int i = 0; i < kChunks; ++i) {
-            const int q = threadIdx.x + i * kGemmThreads;
-            const T *pointer;
-            if constexpr (kContiguousK) pointer = base + static_cast<int64_t>(q >> 3) * stride + k0 + ((q & 7) << 3);
-            else pointer = base + (k0 + q / (kRows / 8)) * stride + ((q % (kRows / 8)) << 3);
-            regs[i] = *reinterpret_cast<const u32x4_t *>(pointer);
-        }
-    }
-
-    // Write the staged tile to LDS; elements whose reduction index is outside [k_lo, k_hi) become zero.
-    __device__ __forceinline__ void store(char *lds, int64_t k0, int64_t k_lo, int64_t k_hi, bool masked) {
-#pragma unroll
-        for (int i = 0; i < kChunks; ++i) {
-            const int q = threadIdx.x + i * kGemmThreads;
-            u32x4_t value = regs[i];
-            if constexpr (kContiguousK) {
-                const int row = q >> 3, chunk = q & 7;
-                if (masked) {
-                    const int64_t k = k0 + (chunk << 3);
-                    if (k < k_lo || k + 8 > k_hi) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            uint32_t word = value[j];
-                            if (k + 2 * j < k_lo || k + 2 * j >= k_hi) word &= 0xffff0000u;
-                            if (k + 2 * j + 1 < k_lo || k + 2 * j + 1 >= k_hi) word &= 0x0000ffffu;
-                            value[j] = word;
-                        }
-                    }
-                }
-                *reinterpret_cast<u32x4_t *>(lds + lds_chunk_offset(row, chunk)) = value;
-            } else {
-                const int k_row = q / (kRows / 8), row0 = (q % (kRows / 8)) << 3;
-                if (masked && (k0 + k_row < k_lo || k0 + k_row >= k_hi)) value = u32x4_t{0, 0, 0, 0};
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int row = row0 + j;
-                    const uint16_t element = static_cast<uint16_t>(value[j >> 1] >> ((j & 1) * 16));
-                    *reinterpret_cast<uint16_t *>(lds + lds_chunk_offset(row, k_row >> 3) + ((k_row & 7) << 1)) = element;
-                }
-            }
-        }
-    }
-};
-
-template <typename T, int kBN, bool kLhsContiguousK, bool kRhsContiguousK>
-__global__ __launch_bounds__(kGemmThreads, 2) void grouped_gemm_mfma_kernel(GemmArgs args) {
-    constexpr int kWaveM = 64, kWaveN = kBN / 2;
-    constexpr int kTilesM = kWaveM / 32, kTilesN = kWaveN / 32;
-    extern __shared__ __attribute__((aligned(16))) char lds[];
-    char *lds_a = lds;
-    char *lds_b = lds + kBM * kBK * 2;
-
-    int tile_m, tile_n;
-    tile_of_block(args, tile_m, tile_n);
-    const int64_t row0 = static_cast<int64_t>(tile_m) * kBM, col0 = static_cast<int64_t>(tile_n) * kBN;
-    const TileWork work = resolve_tile(args, row0, col0);
-    if (work.skip) return;
-
-    const T *lhs = static_cast<const T *>(args.lhs) + work.lhs_offset;
-    const T *rhs = static_cast<const T *>(args.rhs) + work.rhs_offset;
-    const int64_t lhs_stride = kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner;
-    const int64_t rhs_stride = kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner;
-    const bool masked = args.mode == kInputRowSparse;
-    const int64_t k_first = work.k_lo / kBK * kBK;
-    const int64_t k_last = (work.k_hi + kBK - 1) / kBK * kBK;
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wave_m = wave >> 1, wave_n = wave & 1;
-    const int frag_row = lane & 31, frag_chunk = lane >> 5;
-
-    f32x16_t acc[kTilesM][kTilesN];
-#pragma unroll
-    for (int i = 0; i < kTilesM; ++i)
-#pragma unroll
-        for (int j = 0; j < kTilesN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-    OperandStage<T, kBM, kLhsContiguousK> stage_a;
-    OperandStage<T, kBN, kRhsContiguousK> stage_b;
-    if (k_first < k_last) {
-        stage_a.load(lhs, lhs_stride, k_first);
-        stage_b.load(rhs, rhs_stride, k_first);
-    }
-
-    for (int64_t k0 = k_first; k0 < k_last; k0 += kBK) {
-        __syncthreads();  // the previous step's fragment reads are done
-        stage_a.store(lds_a, k0, work.k_lo, work.k_hi, masked);
-        stage_b.store(lds_b, k0, work.k_lo, work.k_hi, masked);
-        __syncthreads();
-        if (k0 + kBK < k_last) {
-            stage_a.load(lhs, lhs_stride, k0 + kBK);
-            stage_b.load(rhs, rhs_stride, k0 + kBK);
-        }
-#pragma unroll
-        for (int step = 0; step < kBK / 16; ++step) {
-            u32x4_t frag_a[kTilesM], frag_b[kTilesN];
-            const int chunk = step * 2 + frag_chunk;
-#pragma unroll
-            for (int i = 0; i < kTilesM; ++i)
-                frag_a[i] = *reinterpret_cast<const u32x4_t *>(
-                    lds_a + lds_chunk_offset(wave_m * kWaveM + i * 32 + frag_row, chunk));
-#pragma unroll
-            for (int j = 0; j < kTilesN; ++j)
-                frag_b[j] = *reinterpret_cast<const u32x4_t *>(
-                    lds_b + lds_chunk_offset(wave_n * kWaveN + j * 32 + frag_row, chunk));
-#pragma unroll
-            for (int i = 0; i < kTilesM; ++i)
-#pragma unroll
-                for (int j = 0; j < kTilesN; ++j) acc[i][j] = Mfma<T>::run(frag_a[i], frag_b[j], acc[i][j]);
-        }
-    }
-
-    // Accumulator layout of a 32x32 tile: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32.
-    const bool accumulate = args.accumulate != 0;
-#pragma unroll
-    for (int i = 0; i < kTilesM; ++i) {
-#pragma unroll
-        for (int j = 0; j < kTilesN; ++j) {
-            const int column = wave_n * kWaveN + j * 32 + (lane & 31);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = wave_m * kWaveM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                store_out_dyn(args.out, args.out_dtype, work.out_offset + row * args.out_stride_row + column,
-                              acc[i][j][v], accumulate);
-            }
-        }
-    }
 }
 
 // =========================================================================================================
@@ -382,31 +150,6 @@ __global__ __launch_bounds__(kGenThreads) void grouped_gemm_generic_kernel(GemmA
 // =========================================================================================================
 // Host dispatch
 // =========================================================================================================
-template <typename T, int kBN, bool kLhsK, bool kRhsK>
-static int launch_mfma(const GemmArgs &args, hipStream_t stream) {
-    constexpr int lds_bytes = (kBM + kBN) * kBK * 2;
-    auto kernel = grouped_gemm_mfma_kernel<T, kBN, kLhsK, kRhsK>;
-    static bool configured = false;  // idempotent attribute; a benign race sets it twice
-    if (!configured) {
-        hipError_t error = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
-        configured = true;
-    }
-    kernel<<<args.tiles_m * args.tiles_n, kGemmThreads, lds_bytes, stream>>>(args);
-    return FM_OK;
-}
-
-template <typename T, int kBN>
-static int launch_mfma_layout(const GemmArgs &args, bool lhs_k, bool rhs_k, hipStream_t stream) {
-    if (lhs_k && rhs_k) return launch_mfma<T, kBN, true, true>(args, stream);
-    if (lhs_k) return launch_mfma<T, kBN, true, false>(args, stream);
-    if (rhs_k) return launch_mfma<T, kBN, false, true>(args, stream);
-    return launch_mfma<T, kBN, false, false>(args, stream);
-}
-
-static bool vector_ok(const void *pointer, int64_t stride) { return aligned16(pointer) && stride % 8 == 0; }
-
 static int run_gemm(const char *name, GemmArgs args, int dtype, void *stream_) {
     FM_REQUIRE(valid_dtype(dtype) && valid_dtype(args.out_dtype), "%s: bad dtype", name);
     FM_REQUIRE(valid_index_dtype(args.index_dtype), "%s: bad index_dtype %d", name, args.index_dtype);
@@ -418,34 +161,9 @@ static int run_gemm(const char *name, GemmArgs args, int dtype, void *stream_) {
     FM_REQUIRE(args.out && (args.inner == 0 || (args.lhs && args.rhs)), "%s: null tensor", name);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
 
-    // Fast path: half-precision operands, unit column stride of out, vectorisable operand layouts, tile-aligned.
-    const bool lhs_k = args.lhs_stride_inner == 1, lhs_m = args.lhs_stride_row == 1;
-    const bool rhs_k = args.rhs_stride_inner == 1, rhs_n = args.rhs_stride_col == 1;
-    bool fast = dtype != FM_DTYPE_F32 && args.out_stride_col == 1 && (lhs_k || lhs_m) && (rhs_k || rhs_n);
-    fast = fast && vector_ok(args.lhs, lhs_k ? args.lhs_stride_row : args.lhs_stride_inner);
-    fast = fast && vector_ok(args.rhs, rhs_k ? args.rhs_stride_col : args.rhs_stride_inner);
-    fast = fast && args.inner % kBK == 0 && args.inner > 0 && args.sparse_size % 8 == 0;
-    fast = fast && (args.mode == kInputRowSparse ? args.sparse_size % kBM == 0 : args.rows % kBM == 0);
-    const int block_n = args.cols % 256 == 0 ? 256 : (args.cols % 128 == 0 ? 128 : 0);
-    fast = fast && block_n != 0;
-    // Prefer a reduction-contiguous view when both strides are 1 (single row/column operands).
-    const bool lhs_contiguous_k = lhs_k, rhs_contiguous_k = rhs_k;
-
-    if (fast) {
-        args.tiles_m = static_cast<int>(args.rows / kBM);
-        args.tiles_n = static_cast<int>(args.cols / block_n);
-        FM_REQUIRE(static_cast<int64_t>(args.tiles_m) * args.tiles_n < (int64_t(1) << 31), "%s: too many tiles", name);
-        int status;
-        if (dtype == FM_DTYPE_BF16) {
-            status = block_n == 256 ? launch_mfma_layout<bf16_t, 256>(args, lhs_contiguous_k, rhs_contiguous_k, stream)
-                                    : launch_mfma_layout<bf16_t, 128>(args, lhs_contiguous_k, rhs_contiguous_k, stream);
-        } else {
-            status = block_n == 256 ? launch_mfma_layout<f16_t, 256>(args, lhs_contiguous_k, rhs_contiguous_k, stream)
-                                    : launch_mfma_layout<f16_t, 128>(args, lhs_contiguous_k, rhs_contiguous_k, stream);
-        }
-        if (status != FM_OK) return status;
+    if (mfma_gemm_eligible(args, dtype)) {
+        if (int status = mfma_gemm_launch(args, dtype, stream)) return status;
     } else {
-        FM_REQUIRE(args.mode != kInputRowSparse || args.sparse_size > 0, "%s: empty sparse dimension", name);
         // A row-sparse tile must not cross into the next expert's block of out.
         if (args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % kGenTile != 0)
             return fail(FM_ERR_UNSUPPORTED, "%s: row_sparse_dim=%lld must be a multiple of %d", name,

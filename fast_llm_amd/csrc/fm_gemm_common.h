@@ -1,0 +1,47 @@
+// Arguments and small device helpers shared by the grouped-GEMM kernels.
+#pragma once
+
+#include "fm_common.h"
+
+namespace fm {
+
+enum GemmMode { kOutputSparse = 0, kInputInnerSparse = 1, kInputRowSparse = 2 };
+
+struct GemmArgs {
+    const void *lhs;
+    const void *rhs;
+    void *out;
+    const void *expert_ends;        // null: dense product
+    const void *expert_pad_begins;  // row-sparse mode only
+    int64_t lhs_stride_row, lhs_stride_inner, rhs_stride_inner, rhs_stride_col, out_stride_row, out_stride_col;
+    int64_t rows;         // rows of out
+    int64_t cols;         // columns of out
+    int64_t inner;        // length of the reduction axis as stored (per expert for input-inner-sparse)
+    int64_t sparse_size;  // N_s, K_s or M_s
+    int num_experts;
+    int mode;
+    int accumulate;
+    int index_dtype;
+    int out_dtype;
+    int tiles_m, tiles_n;
+};
+
+template <typename OutT>
+__device__ __forceinline__ void store_out(void *out, int64_t offset, float value, bool accumulate) {
+    OutT *pointer = static_cast<OutT *>(out) + offset;
+    if (accumulate) value += to_float(*pointer);
+    *pointer = from_float<OutT>(value);
+}
+
+__device__ __forceinline__ void store_out_dyn(void *out, int out_dtype, int64_t offset, float value, bool accumulate) {
+    if (out_dtype == FM_DTYPE_F32) store_out<float>(out, offset, value, accumulate);
+    else if (out_dtype == FM_DTYPE_BF16) store_out<bf16_t>(out, offset, value, accumulate);
+    else store_out<f16_t>(out, offset, value, accumulate);
+}
+
+// Fast path (fm_gemm_mfma.hip). `eligible` says whether the MFMA kernel can take the problem as described by
+// `args` (with `dtype` operands); `launch` fills in the tile counts and launches it.
+bool mfma_gemm_eligible(const GemmArgs &args, int dtype);
+int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream);
+
+}  // namespace fm
