@@ -1,24 +1,29 @@
 // Grouped matrix products on the gfx950 matrix cores (bf16 / fp16 operands, fp32 accumulation).
 //
-// One workgroup = 8 wavefronts = one 256 x 256 tile of `out`, reduced 64 elements of K at a time:
-//   * Operand tiles go from global memory straight into LDS (`global_load_lds_dwordx4`, 16 bytes per lane, no
-//     VGPR staging) into a two-stage ring; the loads of K-step t+1 are in flight while step t is multiplied.
+// One workgroup = 8 wavefronts = one 256 x 256 tile of `out`, reduced one K-slice (kBK elements) at a time:
+//   * A round trip to L2/HBM (~1.5 us under load) takes about two K-slices of multiplying, and LDS only has room
+//     for two 64 KiB slices, so the slices in flight live in registers: every lane keeps two sets of 8 x 16-byte
+//     global loads outstanding (slices t+2 and t+3, 128 KiB per workgroup) while slice t is multiplied from LDS
+//     and slice t+1 is written from registers into the other LDS slot. One barrier per slice.
 //   * An operand may be contiguous along K (activations [rows, K], `weight.t()`) or along its other axis
 //     (`weight` [K, N], `activations.t()`). K-contiguous tiles are stored [row][K] and read as 128-bit MFMA
 //     fragments; the others are stored [K][row] as they lie in memory and read with the LDS transpose load
 //     `ds_read_b64_tr_b16`, which hands every lane four consecutive K values of one row. Both layouts are
-//     XOR-swizzled so that fragment reads hit all 64 banks; the swizzle is applied on the global-address side
-//     because a direct-to-LDS load writes lane i to LDS slot i.
+//     XOR-swizzled so that the 128-bit writes and the fragment reads hit all 64 banks.
 //   * Wavefronts form a 2 x 4 grid, each owns 128 x 64 of the tile as 4 x 2 accumulators of
 //     v_mfma_f32_32x32x16 (128 fp32 registers per lane), two wavefronts per SIMD.
 //   * Tiles never straddle experts: the row tiles of an expert are enumerated from `expert_ends` on the device
 //     (ceil(rows_e / 256) each), a last partial tile loads clamped rows and stores only its valid rows, so any
 //     padding multiple works and phantom rows past the last expert are never touched. For the row-sparse product
-//     the reduction runs over [begin_e, pad_begin_e); a K-tile that sticks out of that range is zeroed in LDS
-//     after it lands (zero-fill, not multiply-by-zero, so NaN in padding rows cannot leak).
+//     the reduction runs over [begin_e, pad_begin_e); what a K-slice holds outside that range is zeroed in LDS
+//     before it is multiplied (zero-fill, not multiply-by-zero, so NaN in padding rows cannot leak).
+//   * The tile is written through LDS: accumulators are laid out row-major per wavefront and stored as 16-byte
+//     vectors, one full 128-byte line of bf16 per row and wavefront.
 //   * Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are renumbered so every XCD works
 //     on a contiguous run of tiles (8 row tiles per column tile) and re-reads operands from its own L2.
 // Results are deterministic: one workgroup per output tile, fixed summation order, no atomics.
+#include <type_traits>
+
 #include "fm_gemm_common.h"
 
 namespace fm {
@@ -29,6 +34,13 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+// Four consecutive output elements, moved as one 8- or 16-byte access.
+template <typename T>
+struct alignas(4 * sizeof(T)) Vec16x4 {
+    T v[4];
+};
 
 #define FM_LDS(T) __attribute__((address_space(3))) T
 #define FM_GLOBAL(T) __attribute__((address_space(1))) T
@@ -50,61 +62,86 @@ struct Mfma<f16_t> {
     }
 };
 
-constexpr int kTile = 256, kBK = 64, kMfmaThreads = 512;
-constexpr int kOperandBytes = kTile * kBK * 2;  // one operand tile in LDS: 32 KiB in either layout
-constexpr int kStageBytes = 2 * kOperandBytes;  // lhs tile, then rhs tile
-constexpr int kStages = 2;
+constexpr int kTile = 256, kMfmaThreads = 512;
+constexpr int kBK = 64;      // K elements per slice (32 or 64)
+constexpr int kStages = 2;   // LDS slots
+constexpr int kOperandBytes = kTile * kBK * 2;  // one operand slice in LDS, same size in either layout
+constexpr int kStageBytes = 2 * kOperandBytes;  // lhs slice, then rhs slice
 constexpr int kLdsBytes = kStages * kStageBytes;
 constexpr int kWaveRows = 128, kWaveCols = 64;  // 2 x 4 wavefronts
+constexpr int kChunksPerRow = kBK / 8;          // 16-byte chunks of a K-major row
+constexpr int kLoadsPerOperand = kBK / 16;      // 16-byte loads per lane, operand and slice
+constexpr int kBufferResourceFlags = 0x00020000;  // raw buffer, 32-bit data format, no swizzle
+constexpr int kEpilogueStride = 72;             // floats per staged row: 64 + padding that keeps 16-byte alignment
+static_assert(kBK == 32 || kBK == 64, "slice width");
+static_assert(kLdsBytes <= 160 * 1024 && 8 * 32 * kEpilogueStride * 4 <= kLdsBytes, "LDS budget");
 
 // ---- LDS layouts ---------------------------------------------------------------------------------------
-// K-contiguous operand, [256 rows][64 k]: 16-byte chunk c (8 k values) of row r sits at r * 128 + ((c ^ ((r >> 1) & 7)) * 16.
+// K-contiguous operand, [256 rows][kBK k]: 16-byte chunk c (8 k values) of row r sits at
+// r * 2 kBK + (c ^ swizzle(r)) * 16 with swizzle(r) = (r / rows-per-256-bytes) mod chunks-per-row.
 // The 16 lanes that read one chunk column of 16 consecutive rows then cover all 64 banks.
-__device__ __forceinline__ int lds_offset_k_major(int row, int chunk) {
-    return row * (kBK * 2) + ((chunk ^ ((row >> 1) & 7)) << 4);
+__device__ __forceinline__ int k_major_swizzle(int row) {
+    return (row / (128 / kBK)) & (kChunksPerRow - 1);
 }
-// Row-contiguous operand, [64 k][256 rows]: the 32-byte group g (16 rows) of K-row k sits at k * 512 + (g ^ (2 * (k & 3))) * 32.
+__device__ __forceinline__ int lds_offset_k_major(int row, int chunk) {
+    return row * (kBK * 2) + ((chunk ^ k_major_swizzle(row)) << 4);
+}
+// Row-contiguous operand, [kBK k][256 rows]: the 32-byte group g (16 rows) of K-row k sits at k * 512 + (g ^ (2 * (k & 3))) * 32.
 // A transpose load by 32 lanes touches 4 K-rows x 2 groups; the XOR sends them to 8 different bank octets.
 __device__ __forceinline__ int lds_offset_row_major(int k, int row) {
     return k * (kTile * 2) + ((((row >> 4) ^ ((k & 3) << 1)) << 5) | ((row & 15) << 1));
 }
 
-// Direct global -> LDS loader of one operand tile per K-step. Each of the 8 wavefronts issues 4 loads of
-// 64 lanes x 16 bytes; load j of wavefront w fills LDS slots [(4 w + j) * 64, +64) of the operand tile.
+// Loader of one operand slice: global memory -> registers -> LDS. The slice is 256 * kBK / 8 chunks of 16 bytes;
+// chunk slot p of the LDS slice is handled by lane p % 64 of wavefront (p / 64) / kLoadsPerOperand as its load
+// number (p / 64) % kLoadsPerOperand, so a wavefront writes 1 KiB of consecutive LDS per instruction.
 template <bool kContiguousK>
 struct TileLoader {
-    const char *pointer[4];
-    int64_t step;
+    const char *base;                   // wave-uniform: first row of the tile, first k of the current slice
+    uint32_t offset[kLoadsPerOperand];  // per lane, bytes from `base` (fits 32 bits: checked on the host)
+    int64_t step;                       // bytes from one slice to the next
+    int lds_offset;                     // of this lane's first slot
 
-    // `base`: element (first row of the tile, first k of the loop). `stride`: bytes between rows (K-contiguous)
-    // or between K-rows (row-contiguous). Rows >= valid_rows are replaced by in-range ones (never stored).
-    __device__ __forceinline__ void setup(const char *base, int64_t stride, int valid_rows, int wave, int lane) {
+    // `stride`: bytes between rows (K-contiguous) or between K-rows (row-contiguous). Rows >= valid_rows are
+    // replaced by in-range ones (their products are never stored).
+    __device__ __forceinline__ void setup(const char *tile_base, int64_t stride, int valid_rows, int wave, int lane) {
+        base = tile_base;
+        lds_offset = (wave * kLoadsPerOperand * 64 + lane) * 16;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int slot = (wave * 4 + j) * 64 + lane;
+        for (int j = 0; j < kLoadsPerOperand; ++j) {
+            const int slot = (wave * kLoadsPerOperand + j) * 64 + lane;
             if constexpr (kContiguousK) {
-                const int row = slot >> 3;
-                const int chunk = (slot & 7) ^ ((row >> 1) & 7);
-                pointer[j] = base + static_cast<int64_t>(min(row, valid_rows - 1)) * stride + chunk * 16;
+                const int row = slot / kChunksPerRow;
+                const int chunk = (slot % kChunksPerRow) ^ k_major_swizzle(row);
+                offset[j] = static_cast<uint32_t>(min(row, valid_rows - 1) * stride + chunk * 16);
             } else {
                 const int k = slot >> 5, position = slot & 31;
                 const int group = (position >> 1) ^ ((k & 3) << 1);
                 int first_row = (group * 2 + (position & 1)) * 8;
                 if (first_row >= valid_rows) first_row = 0;
-                pointer[j] = base + k * stride + first_row * 2;
+                offset[j] = static_cast<uint32_t>(k * stride + first_row * 2);
             }
         }
         step = kContiguousK ? kBK * 2 : kBK * stride;
     }
 
-    __device__ __forceinline__ void issue(FM_LDS(char) * operand_lds, int wave) {
+    // Buffer loads: scalar base (in the resource descriptor) + 32-bit lane offset, so the addresses cost one
+    // register per load and advancing to the next slice is scalar arithmetic.
+    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand]) {
+        const __amdgpu_buffer_rsrc_t resource =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, -1, kBufferResourceFlags);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            __builtin_amdgcn_global_load_lds((const FM_GLOBAL(void) *)(pointer[j]),
-                                             reinterpret_cast<FM_LDS(void) *>(operand_lds + (wave * 4 + j) * 1024), 16,
-                                             0, 0);
-            pointer[j] += step;
-        }
+        for (int j = 0; j < kLoadsPerOperand; ++j)
+            regs[j] = __builtin_bit_cast(
+                u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, static_cast<int>(offset[j]), 0, 0));
+        base += step;
+    }
+
+    // Write a landed slice into LDS.
+    __device__ __forceinline__ void store(const u32x4_t (&regs)[kLoadsPerOperand], FM_LDS(char) * operand_lds) {
+#pragma unroll
+        for (int j = 0; j < kLoadsPerOperand; ++j)
+            *reinterpret_cast<FM_LDS(u32x4_t) *>(operand_lds + lds_offset + j * 1024) = regs[j];
     }
 };
 
@@ -130,26 +167,27 @@ __device__ __forceinline__ u32x4_t load_fragment(FM_LDS(char) * operand_lds, int
     }
 }
 
-// Zero, in a landed LDS tile whose K origin is k0, everything whose reduction index is outside [k_lo, k_hi).
+// Zero, in a slice that sits in LDS and whose first reduction index is k0, everything whose reduction index is
+// outside [k_lo, k_hi). Runs between two barriers, for the first/last slice of a ragged reduction range only.
 template <bool kContiguousK>
-__device__ __forceinline__ void mask_tile(FM_LDS(char) * operand_lds, int64_t k0, int64_t k_lo, int64_t k_hi) {
+__device__ __forceinline__ void mask_tile(FM_LDS(char) * operand_lds, int k0, int k_lo, int k_hi) {
     for (int slot = threadIdx.x; slot < kOperandBytes / 16; slot += kMfmaThreads) {
         FM_LDS(u32x4_t) *pointer = reinterpret_cast<FM_LDS(u32x4_t) *>(operand_lds + slot * 16);
         if constexpr (kContiguousK) {
-            const int row = slot >> 3;
-            const int64_t k = k0 + (((slot & 7) ^ ((row >> 1) & 7)) << 3);
+            const int row = slot / kChunksPerRow;
+            const int k = k0 + (((slot % kChunksPerRow) ^ k_major_swizzle(row)) << 3);
             if (k >= k_lo && k + 8 <= k_hi) continue;
             u32x4_t value = *pointer;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                uint32_t word = value[j];
-                if (k + 2 * j < k_lo || k + 2 * j >= k_hi) word &= 0xffff0000u;
-                if (k + 2 * j + 1 < k_lo || k + 2 * j + 1 >= k_hi) word &= 0x0000ffffu;
-                value[j] = word;
+            for (int w = 0; w < 4; ++w) {
+                uint32_t word = value[w];
+                if (k + 2 * w < k_lo || k + 2 * w >= k_hi) word &= 0xffff0000u;
+                if (k + 2 * w + 1 < k_lo || k + 2 * w + 1 >= k_hi) word &= 0x0000ffffu;
+                value[w] = word;
             }
             *pointer = value;
         } else {
-            const int64_t k = k0 + (slot >> 5);
+            const int k = k0 + (slot >> 5);
             if (k < k_lo || k >= k_hi) *pointer = u32x4_t{0, 0, 0, 0};
         }
     }
@@ -258,30 +296,64 @@ __device__ __forceinline__ void tile_of_block(const GemmArgs &args, int &tile_m,
 }
 
 // ---- the kernel ----------------------------------------------------------------------------------------
+// Tell the compiler that a pointer computed from tile coordinates is the same in every lane (it then lives in
+// scalar registers and the loads use the scalar-base addressing form).
+__device__ __forceinline__ const char *uniform_pointer(const char *pointer) {
+    const uint64_t bits = reinterpret_cast<uint64_t>(pointer);
+    const uint32_t low = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+    const uint32_t high = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+    return reinterpret_cast<const char *>((static_cast<uint64_t>(high) << 32) | low);
+}
+
+// Write the wavefront's 128 x 64 accumulators through its own LDS region, 32 rows at a time: registers -> LDS as
+// [32][kEpilogueStride] floats, then every lane takes 4 consecutive columns, so one store instruction covers 4 rows
+// x 64 columns (full 128-byte lines for 2-byte outputs). Row stride 72 floats keeps both the scalar writes (two
+// row groups 4 rows apart per instruction) and the 16-byte reads free of bank conflicts.
 template <typename OutT>
-__device__ __forceinline__ void store_tile(const f32x16_t (&acc)[4][2], OutT *out, int64_t stride, int rows_valid,
-                                           int cols_valid, bool accumulate, int wave_m, int wave_n, int lane) {
-    // Accumulator register v of lane l in a 32x32 tile: row 8 (v / 4) + 4 (l / 32) + v % 4, column l % 32.
+__device__ __forceinline__ void store_tile(const f32x16_t (&acc)[4][2], FM_LDS(char) * lds, OutT *out, int64_t stride,
+                                           int rows_valid, int cols_valid, bool accumulate, int wave, int lane) {
+    const int wave_m = wave >> 2, wave_n = wave & 3;
+    FM_LDS(float) *staging = reinterpret_cast<FM_LDS(float) *>(lds) + wave * (32 * kEpilogueStride);
+    const int column = (lane & 15) * 4;  // within the wavefront's 64 columns
+    const int column_in_tile = wave_n * kWaveCols + column;
+    // cols_valid is a multiple of 8, so a group of 4 columns is valid or not as a whole.
+    const bool column_ok = column_in_tile < cols_valid;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int column = wave_n * kWaveCols + j * 32 + (lane & 31);
-            if (column >= cols_valid) continue;
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = wave_m * kWaveRows + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row >= rows_valid) continue;
-                OutT *pointer = out + row * stride + column;
-                float value = acc[i][j][v];
-                if (accumulate) value += to_float(*pointer);
-                *pointer = from_float<OutT>(value);
+            for (int v = 0; v < 16; ++v)
+                staging[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * kEpilogueStride + j * 32 + (lane & 31)] =
+                    acc[i][j][v];
+        // Only this wavefront touches its staging region and the LDS executes a wavefront's operations in order,
+        // so no barrier is needed; the empty asm only keeps the compiler from moving accesses across the phases.
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int staged_row = t * 4 + (lane >> 4);
+            const int row = wave_m * kWaveRows + i * 32 + staged_row;
+            const f32x4_t value = *reinterpret_cast<FM_LDS(f32x4_t) *>(staging + staged_row * kEpilogueStride + column);
+            if (row < rows_valid && column_ok) {
+                Vec16x4<OutT> packed;
+                OutT *pointer = out + row * stride + column_in_tile;
+                if (accumulate) {
+                    packed = *reinterpret_cast<const Vec16x4<OutT> *>(pointer);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) packed.v[c] = from_float<OutT>(value[c] + to_float(packed.v[c]));
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) packed.v[c] = from_float<OutT>(value[c]);
+                }
+                *reinterpret_cast<Vec16x4<OutT> *>(pointer) = packed;
             }
         }
+        asm volatile("" ::: "memory");
     }
 }
 
-template <typename T, bool kLhsContiguousK, bool kRhsContiguousK>
+// kMasked: the row-sparse product, whose reduction range [k_lo, k_hi) is ragged.
+template <typename T, bool kLhsContiguousK, bool kRhsContiguousK, bool kMasked>
 __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(GemmArgs args) {
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);  // C-style: address-space cast
@@ -294,10 +366,14 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wave_m = wave >> 2, wave_n = wave & 3;
-    const bool masked = args.mode == kInputRowSparse;
+    // Tile coordinates are the same in every lane; say so, so that they live in scalar registers.
+    work.k_lo = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_lo));
+    work.k_hi = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_hi));
+    work.rows_valid = __builtin_amdgcn_readfirstlane(work.rows_valid);
+    work.cols_valid = __builtin_amdgcn_readfirstlane(work.cols_valid);
     const int64_t k_first = work.k_lo / kBK * kBK;
     const int64_t k_last = work.k_hi > work.k_lo ? (work.k_hi + kBK - 1) / kBK * kBK : k_first;
-    const int num_steps = static_cast<int>((k_last - k_first) / kBK);
+    const int num_slices = __builtin_amdgcn_readfirstlane(static_cast<int>((k_last - k_first) / kBK));
 
     TileLoader<kLhsContiguousK> load_lhs;
     TileLoader<kRhsContiguousK> load_rhs;
@@ -306,9 +382,9 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
                           (work.lhs_offset + k_first * args.lhs_stride_inner) * static_cast<int64_t>(sizeof(T));
         const char *rhs = static_cast<const char *>(args.rhs) +
                           (work.rhs_offset + k_first * args.rhs_stride_inner) * static_cast<int64_t>(sizeof(T));
-        load_lhs.setup(lhs, (kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner) * sizeof(T),
+        load_lhs.setup(uniform_pointer(lhs), (kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner) * sizeof(T),
                        work.rows_valid, wave, lane);
-        load_rhs.setup(rhs, (kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner) * sizeof(T),
+        load_rhs.setup(uniform_pointer(rhs), (kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner) * sizeof(T),
                        work.cols_valid, wave, lane);
     }
 
@@ -320,63 +396,99 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    if (num_steps > 0) {
-        load_lhs.issue(lds, wave);
-        load_rhs.issue(lds + kOperandBytes, wave);
-    }
-    for (int step = 0; step < num_steps; ++step) {
-        FM_LDS(char) *stage = lds + (step & 1) * kStageBytes;
-        // This wavefront's loads of `stage` have landed; after the barrier everybody's have, and everybody is done
-        // reading the other stage, which the next loads overwrite.
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (masked) {
-            const int64_t k0 = k_first + static_cast<int64_t>(step) * kBK;
-            if (k0 < work.k_lo || k0 + kBK > work.k_hi) {
-                mask_tile<kLhsContiguousK>(stage, k0, work.k_lo, work.k_hi);
-                mask_tile<kRhsContiguousK>(stage + kOperandBytes, k0, work.k_lo, work.k_hi);
-                __syncthreads();
-            }
-        }
-        if (step + 1 < num_steps) {
-            FM_LDS(char) *next = lds + ((step + 1) & 1) * kStageBytes;
-            load_lhs.issue(next, wave);
-            load_rhs.issue(next + kOperandBytes, wave);
-        }
+    // Register sets 0/1 hold the slices in flight; slice s travels in set s % 2 and ends in LDS slot s % 2.
+    u32x4_t lhs_regs[2][kLoadsPerOperand], rhs_regs[2][kLoadsPerOperand];
+    auto stage_of = [&](int slice) { return lds + (slice & 1) * kStageBytes; };
+    auto write_slice = [&](int slice, auto set) {
+        load_lhs.store(lhs_regs[set], stage_of(slice));
+        load_rhs.store(rhs_regs[set], stage_of(slice) + kOperandBytes);
+    };
+    auto fetch_slice = [&](auto set) {
+        load_lhs.load(lhs_regs[set]);
+        load_rhs.load(rhs_regs[set]);
+    };
+    auto multiply_slice = [&](int slice) {
+        FM_LDS(char) *stage = stage_of(slice);
 #pragma unroll
         for (int kstep = 0; kstep < kBK / 16; ++kstep) {
-            u32x4_t frag_a[4], frag_b[2];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                frag_a[i] = load_fragment<kLhsContiguousK>(stage, wave_m * kWaveRows + i * 32, kstep, lane);
+            u32x4_t frag_b[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 frag_b[j] =
                     load_fragment<kRhsContiguousK>(stage + kOperandBytes, wave_n * kWaveCols + j * 32, kstep, lane);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < 4; ++i) {
+                const u32x4_t frag_a = load_fragment<kLhsContiguousK>(stage, wave_m * kWaveRows + i * 32, kstep, lane);
 #pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(frag_a[i], frag_b[j], acc[i][j]);
+                for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(frag_a, frag_b[j], acc[i][j]);
+            }
         }
+    };
+    // One iteration: after the barrier slice t is visible in LDS slot t % 2 and slot (t + 1) % 2 is free. Slice
+    // t + 1 (in flight for two iterations) goes from its register set to that slot, the set is refilled with
+    // slice t + 3, then slice t is multiplied while t + 2 and t + 3 are in flight.
+    // `steady`: slices t + 1 and t + 3 exist, nothing is conditional. The compiler places the `s_waitcnt vmcnt`
+    // that guards a register set; only where every load on the way is unconditional does it know that 8 newer
+    // loads are outstanding and waits with vmcnt(8..15) instead of draining the queue, so the steady-state loop and
+    // the prologue that leads into it are kept free of branches around loads.
+    auto iteration = [&](int t, auto next_set, auto steady) {
+        __syncthreads();
+        if constexpr (kMasked) {
+            const int k0 = static_cast<int>(k_first) + t * kBK;
+            if (k0 < work.k_lo || k0 + kBK > work.k_hi) {  // wave-uniform: first/last slice of the range
+                mask_tile<kLhsContiguousK>(stage_of(t), k0, work.k_lo, work.k_hi);
+                mask_tile<kRhsContiguousK>(stage_of(t) + kOperandBytes, k0, work.k_lo, work.k_hi);
+                __syncthreads();
+            }
+        }
+        if (decltype(steady)::value || t + 1 < num_slices) write_slice(t + 1, next_set);
+        if (decltype(steady)::value || t + 3 < num_slices) fetch_slice(next_set);
+        // Keep the scheduler from sinking the loads into the multiply: they must be issued first to get two full
+        // iterations of flight time.
+        __builtin_amdgcn_sched_barrier(0);
+        multiply_slice(t);
+    };
+    constexpr std::integral_constant<int, 0> set0{};
+    constexpr std::integral_constant<int, 1> set1{};
+    int t = 0;
+    if (num_slices >= 5) {
+        fetch_slice(set0);
+        fetch_slice(set1);
+        write_slice(0, set0);
+        fetch_slice(set0);
+        for (; t + 4 < num_slices; t += 2) {  // slices up to t + 4 exist
+            iteration(t, set1, std::true_type{});
+            iteration(t + 1, set0, std::true_type{});
+        }
+    } else {
+        if (num_slices > 0) fetch_slice(set0);
+        if (num_slices > 1) fetch_slice(set1);
+        if (num_slices > 0) write_slice(0, set0);
+        if (num_slices > 2) fetch_slice(set0);
+    }
+    for (; t < num_slices; t += 2) {  // the last (at most four) slices
+        iteration(t, set1, std::false_type{});
+        if (t + 1 < num_slices) iteration(t + 1, set0, std::false_type{});
     }
 
     const bool accumulate = args.accumulate != 0;
-    if (accumulate && num_steps == 0) return;  // nothing to add
+    if (accumulate && num_slices == 0) return;  // nothing to add
+    __syncthreads();  // all wavefronts are done reading operand slices; LDS becomes the staging area
     if (args.out_dtype == FM_DTYPE_F32)
-        store_tile(acc, static_cast<float *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
-                   work.cols_valid, accumulate, wave_m, wave_n, lane);
+        store_tile(acc, lds, static_cast<float *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
+                   work.cols_valid, accumulate, wave, lane);
     else if (args.out_dtype == FM_DTYPE_BF16)
-        store_tile(acc, static_cast<bf16_t *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
-                   work.cols_valid, accumulate, wave_m, wave_n, lane);
+        store_tile(acc, lds, static_cast<bf16_t *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
+                   work.cols_valid, accumulate, wave, lane);
     else
-        store_tile(acc, static_cast<f16_t *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
-                   work.cols_valid, accumulate, wave_m, wave_n, lane);
+        store_tile(acc, lds, static_cast<f16_t *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
+                   work.cols_valid, accumulate, wave, lane);
 }
 
 // ---- host side -----------------------------------------------------------------------------------------
-template <typename T, bool kLhsK, bool kRhsK>
+template <typename T, bool kLhsK, bool kRhsK, bool kMasked>
 static int launch_instance(const GemmArgs &args, hipStream_t stream) {
-    auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK>;
+    auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK, kMasked>;
     static bool configured = false;  // setting the attribute twice from racing threads is harmless
     if (!configured) {
         hipError_t error = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -391,10 +503,15 @@ static int launch_instance(const GemmArgs &args, hipStream_t stream) {
 template <typename T>
 static int launch_layout(const GemmArgs &args, hipStream_t stream) {
     const bool lhs_k = args.lhs_stride_inner == 1, rhs_k = args.rhs_stride_inner == 1;
-    if (lhs_k && rhs_k) return launch_instance<T, true, true>(args, stream);
-    if (lhs_k) return launch_instance<T, true, false>(args, stream);
-    if (rhs_k) return launch_instance<T, false, true>(args, stream);
-    return launch_instance<T, false, false>(args, stream);
+    // Only the row-sparse product with a map has a ragged reduction range.
+    const bool masked = args.mode == kInputRowSparse && args.expert_ends != nullptr;
+#define FM_LAUNCH(LHS, RHS) \
+    return masked ? launch_instance<T, LHS, RHS, true>(args, stream) : launch_instance<T, LHS, RHS, false>(args, stream)
+    if (lhs_k && rhs_k) FM_LAUNCH(true, true);
+    if (lhs_k) FM_LAUNCH(true, false);
+    if (rhs_k) FM_LAUNCH(false, true);
+    FM_LAUNCH(false, false);
+#undef FM_LAUNCH
 }
 
 static bool vector_ok(const void *pointer, int64_t stride) { return aligned16(pointer) && stride % 8 == 0; }
@@ -410,6 +527,12 @@ bool mfma_gemm_eligible(const GemmArgs &args, int dtype) {
     // contiguous axis of a row-contiguous operand must not straddle the end of an expert's block.
     if (args.inner <= 0 || args.inner % kBK != 0 || args.sparse_size % 8 != 0 || args.cols % 8 != 0) return false;
     if (!lhs_k && args.mode != kInputRowSparse && args.rows % 8 != 0) return false;
+    // Per-lane byte offsets inside an operand tile are 32-bit.
+    if (max(max(args.lhs_stride_row, args.lhs_stride_inner), max(args.rhs_stride_inner, args.rhs_stride_col)) >=
+        (int64_t(1) << 21))
+        return false;
+    // The tile is stored as vectors of 4 elements.
+    if (!aligned16(args.out) || args.out_stride_row % 8 != 0) return false;
     return true;
 }
 
