@@ -14,6 +14,7 @@ bandwidth-bound kernels, and a CPU baseline (the looped torch MoE on the host co
 import argparse
 import json
 import os
+import pathlib
 import sys
 import time
 
@@ -21,6 +22,19 @@ import torch
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E peak, GB/s
+# HBM traffic per GEMM launch cannot be measured from inside the process; it comes from the committed summary of two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, WRITE_SIZE, calibrated on the copy kernel below).
+TRAFFIC_SUMMARY = pathlib.Path(__file__).resolve().parent / "profiles" / "bench_mixtral_hbm_traffic.json"
+
+
+def measured_traffic(workload_name: str) -> tuple[int | None, str | None]:
+    try:
+        summary = json.loads(TRAFFIC_SUMMARY.read_text())
+    except (OSError, ValueError):
+        return None, None
+    if summary.get("workload") != workload_name:
+        return None, None
+    return summary["traffic_bytes_per_launch"], summary["source"]
 
 
 def parse_args() -> argparse.Namespace:
@@ -32,6 +46,13 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--recompute", default="none", help="none | activation | activation_and_input | full")
     parser.add_argument("--cpu-tokens", type=int, default=512, help="tokens in the CPU baseline sample (0: skip)")
     parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument(
+        "--calibration-mib",
+        type=int,
+        default=1024,
+        help="size of a plain device copy done once before the warm-up; hardware counters (FETCH_SIZE, WRITE_SIZE) "
+        "read for it calibrate the counters read for the kernels of the timed region (0: skip)",
+    )
     return parser.parse_args()
 
 
@@ -105,6 +126,12 @@ def main() -> None:
         )
         output.backward(inputs.grad_output)
 
+    if args.calibration_mib > 0:
+        # One read and one write of a known size, outside the timed region: an elementwise add kernel (a plain
+        # `copy_` would go through the runtime's blit path, for which no counters are reported).
+        source = torch.ones(args.calibration_mib << 18, dtype=torch.float32, device=device)
+        torch.add(source, 1.0, out=torch.empty_like(source))
+        del source
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -123,6 +150,7 @@ def main() -> None:
     rows, hidden, ffn = workload.sparse_rows_unpadded, workload.hidden, workload.ffn
     itemsize = workload.dtype.itemsize
     gemm_ms = sum(durations[label] * calls_per_step[label] for label in durations if "matmul" in label)
+    gemm_launches = sum(calls_per_step[label] for label in durations if "matmul" in label)
     gemm_flops = workload.gemm_flops * (4 / 3 if recompute_level.recompute_layer_1 else 1)
     gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
     index_size = 2 if rows + workload.experts * 128 < 32768 else 4
@@ -149,6 +177,7 @@ def main() -> None:
             entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
         kernels[label] = entry
 
+    traffic, traffic_source = measured_traffic(workload.name)
     result = {
         "metric": "MoE fwd+bwd tokens/s at Mixtral shape; grouped-GEMM % bf16 MFMA peak",
         "value": tokens_per_second,
@@ -174,14 +203,16 @@ def main() -> None:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "grouped_gemm_mfma_kernel (six launches per step)",
+            "kernel": "grouped_gemm_mfma_kernel (all grouped-GEMM launches of a step; figures are per launch, averaged over them)",
             "achieved": gemm_tflops,
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_tflops / PEAK_BF16_TFLOPS,
-            "traffic": None,
-            "flops_per_step": gemm_flops,
-            "ms_per_step": gemm_ms,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
+            "launches_per_step": gemm_launches,
+            "flops_per_launch": gemm_flops / gemm_launches,
+            "ms_per_launch": gemm_ms / gemm_launches,
         },
         "gemm_frac_of_step": gemm_ms / ms_per_step,
         "kernels": kernels,
