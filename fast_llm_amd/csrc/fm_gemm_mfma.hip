@@ -73,7 +73,7 @@ constexpr int kChunksPerRow = kBK / 8;          // 16-byte chunks of a K-major r
 constexpr int kLoadsPerOperand = kBK / 16;      // 16-byte loads per lane, operand and slice
 constexpr int kBufferResourceFlags = 0x00020000;  // raw buffer, 32-bit data format, no swizzle
 constexpr int kEpilogueStride = 72;             // floats per staged row: 64 + padding that keeps 16-byte alignment
-static_assert(kBK == 32 || kBK == 64, "slice width");
+static_assert(kBK == 64, "slice width: the pipeline spreads kLoadsPerOperand = 4 chunks over the 4 K-steps of a slice");
 static_assert(kLdsBytes <= 160 * 1024 && 8 * 32 * kEpilogueStride * 4 <= kLdsBytes, "LDS budget");
 
 // ---- LDS layouts ---------------------------------------------------------------------------------------
@@ -127,21 +127,28 @@ struct TileLoader {
 
     // Buffer loads: scalar base (in the resource descriptor) + 32-bit lane offset, so the addresses cost one
     // register per load and advancing to the next slice is scalar arithmetic.
-    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand]) {
+    // Load j of the current slice; `advance` moves on to the next slice (after its last load).
+    __device__ __forceinline__ void load_one(u32x4_t (&regs)[kLoadsPerOperand], int j) {
         const __amdgpu_buffer_rsrc_t resource =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, -1, kBufferResourceFlags);
+        regs[j] = __builtin_bit_cast(
+            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, static_cast<int>(offset[j]), 0, 0));
+    }
+    __device__ __forceinline__ void advance() { base += step; }
+    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand]) {
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j)
-            regs[j] = __builtin_bit_cast(
-                u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, static_cast<int>(offset[j]), 0, 0));
-        base += step;
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_one(regs, j);
+        advance();
     }
 
-    // Write a landed slice into LDS.
+    // Write a landed slice (or its chunk j) into LDS.
+    __device__ __forceinline__ void store_one(const u32x4_t (&regs)[kLoadsPerOperand], FM_LDS(char) * operand_lds,
+                                              int j) {
+        *reinterpret_cast<FM_LDS(u32x4_t) *>(operand_lds + lds_offset + j * 1024) = regs[j];
+    }
     __device__ __forceinline__ void store(const u32x4_t (&regs)[kLoadsPerOperand], FM_LDS(char) * operand_lds) {
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j)
-            *reinterpret_cast<FM_LDS(u32x4_t) *>(operand_lds + lds_offset + j * 1024) = regs[j];
+        for (int j = 0; j < kLoadsPerOperand; ++j) store_one(regs, operand_lds, j);
     }
 };
 
@@ -407,8 +414,12 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
         load_lhs.load(lhs_regs[set]);
         load_rhs.load(rhs_regs[set]);
     };
-    auto multiply_slice = [&](int slice) {
+    // Multiply slice `slice` from LDS. With `steady`, the traffic for the slices behind it is spread over the four
+    // K-steps instead of being a burst after the barrier: chunk q of slice + 1 goes from register set `set` to LDS
+    // and the freed registers are refilled with chunk q of slice + 3, while the MFMAs of K-step q run.
+    auto multiply_slice = [&](int slice, auto set, auto steady) {
         FM_LDS(char) *stage = stage_of(slice);
+        FM_LDS(char) *next_stage = stage_of(slice + 1);
 #pragma unroll
         for (int kstep = 0; kstep < kBK / 16; ++kstep) {
             u32x4_t frag_b[2];
@@ -416,12 +427,25 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
             for (int j = 0; j < 2; ++j)
                 frag_b[j] =
                     load_fragment<kRhsContiguousK>(stage + kOperandBytes, wave_n * kWaveCols + j * 32, kstep, lane);
+            if constexpr (decltype(steady)::value) {
+                load_lhs.store_one(lhs_regs[set], next_stage, kstep);
+                load_rhs.store_one(rhs_regs[set], next_stage + kOperandBytes, kstep);
+                load_lhs.load_one(lhs_regs[set], kstep);
+                load_rhs.load_one(rhs_regs[set], kstep);
+                if (kstep == kBK / 16 - 1) {
+                    load_lhs.advance();
+                    load_rhs.advance();
+                }
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const u32x4_t frag_a = load_fragment<kLhsContiguousK>(stage, wave_m * kWaveRows + i * 32, kstep, lane);
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(frag_a, frag_b[j], acc[i][j]);
             }
+            // One K-step is one scheduling region: the compiler may interleave inside it but not merge the memory
+            // traffic of several K-steps into one burst.
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     // One iteration: after the barrier slice t is visible in LDS slot t % 2 and slot (t + 1) % 2 is free. Slice
@@ -441,12 +465,13 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
                 __syncthreads();
             }
         }
-        if (decltype(steady)::value || t + 1 < num_slices) write_slice(t + 1, next_set);
-        if (decltype(steady)::value || t + 3 < num_slices) fetch_slice(next_set);
-        // Keep the scheduler from sinking the loads into the multiply: they must be issued first to get two full
-        // iterations of flight time.
-        __builtin_amdgcn_sched_barrier(0);
-        multiply_slice(t);
+        if constexpr (decltype(steady)::value) {
+            multiply_slice(t, next_set, std::true_type{});
+        } else {
+            if (t + 1 < num_slices) write_slice(t + 1, next_set);
+            if (t + 3 < num_slices) fetch_slice(next_set);
+            multiply_slice(t, next_set, std::false_type{});
+        }
     };
     constexpr std::integral_constant<int, 0> set0{};
     constexpr std::integral_constant<int, 1> set1{};
