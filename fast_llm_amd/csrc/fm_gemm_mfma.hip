@@ -1,17 +1,20 @@
 // Grouped matrix products on the gfx950 matrix cores (bf16 / fp16 operands, fp32 accumulation).
 //
-// One workgroup = 8 wavefronts = one 256 x 256 tile of `out`, reduced one K-slice (kBK elements) at a time:
+// One workgroup = 4 wavefronts = one 256 x 256 tile of `out`, reduced one K-slice (kBK = 64 elements) at a time:
 //   * A round trip to L2/HBM (~1.5 us under load) takes about two K-slices of multiplying, and LDS only has room
-//     for two 64 KiB slices, so the slices in flight live in registers: every lane keeps two sets of 8 x 16-byte
+//     for two 64 KiB slices, so the slices in flight live in registers: every lane keeps two sets of 16 x 16-byte
 //     global loads outstanding (slices t+2 and t+3, 128 KiB per workgroup) while slice t is multiplied from LDS
-//     and slice t+1 is written from registers into the other LDS slot. One barrier per slice.
+//     and slice t+1 is written from registers into the other LDS slot. One barrier per slice, placed before the last
+//     K-step of a slice, whose MFMAs overlap the first fragment reads of the next slice.
 //   * An operand may be contiguous along K (activations [rows, K], `weight.t()`) or along its other axis
 //     (`weight` [K, N], `activations.t()`). K-contiguous tiles are stored [row][K] and read as 128-bit MFMA
 //     fragments; the others are stored [K][row] as they lie in memory and read with the LDS transpose load
 //     `ds_read_b64_tr_b16`, which hands every lane four consecutive K values of one row. Both layouts are
 //     XOR-swizzled so that the 128-bit writes and the fragment reads hit all 64 banks.
-//   * Wavefronts form a 2 x 4 grid, each owns 128 x 64 of the tile as 4 x 2 accumulators of
-//     v_mfma_f32_32x32x16 (128 fp32 registers per lane), two wavefronts per SIMD.
+//   * Wavefronts form a 2 x 2 grid, one per SIMD, each owns 128 x 128 of the tile as 4 x 4 accumulators of
+//     v_mfma_f32_32x32x16 (256 accumulation registers per lane; the other 256 hold the in-flight slices and the
+//     fragments). A single wavefront keeps the matrix pipe busy as long as its MFMAs are back to back, so every
+//     K-step is scheduled as "one MFMA, one memory instruction in its shadow" (sched_group_barrier).
 //   * Tiles never straddle experts: the row tiles of an expert are enumerated from `expert_ends` on the device
 //     (ceil(rows_e / 256) each), a last partial tile loads clamped rows and stores only its valid rows, so any
 //     padding multiple works and phantom rows past the last expert are never touched. For the row-sparse product
@@ -62,19 +65,24 @@ struct Mfma<f16_t> {
     }
 };
 
-constexpr int kTile = 256, kMfmaThreads = 512;
+constexpr int kTile = 256;
+constexpr int kWavesM = 2, kWavesN = 2;  // wavefront grid over the tile
+constexpr int kWaves = kWavesM * kWavesN, kMfmaThreads = 64 * kWaves;
 constexpr int kBK = 64;      // K elements per slice (32 or 64)
 constexpr int kStages = 2;   // LDS slots
 constexpr int kOperandBytes = kTile * kBK * 2;  // one operand slice in LDS, same size in either layout
 constexpr int kStageBytes = 2 * kOperandBytes;  // lhs slice, then rhs slice
 constexpr int kLdsBytes = kStages * kStageBytes;
-constexpr int kWaveRows = 128, kWaveCols = 64;  // 2 x 4 wavefronts
+constexpr int kWaveRows = kTile / kWavesM, kWaveCols = kTile / kWavesN;  // a wavefront's part of the tile
+constexpr int kTilesM = kWaveRows / 32, kTilesN = kWaveCols / 32;        // in 32x32 MFMA accumulators
 constexpr int kChunksPerRow = kBK / 8;          // 16-byte chunks of a K-major row
-constexpr int kLoadsPerOperand = kBK / 16;      // 16-byte loads per lane, operand and slice
+constexpr int kLoadsPerOperand = kOperandBytes / 16 / kMfmaThreads;  // 16-byte loads per lane, operand and slice
+constexpr int kLoadsPerStep = kLoadsPerOperand / (kBK / 16);        // of them moved during one K-step
 constexpr int kBufferResourceFlags = 0x00020000;  // raw buffer, 32-bit data format, no swizzle
-constexpr int kEpilogueStride = 72;             // floats per staged row: 64 + padding that keeps 16-byte alignment
-static_assert(kBK == 64, "slice width: the pipeline spreads kLoadsPerOperand = 4 chunks over the 4 K-steps of a slice");
-static_assert(kLdsBytes <= 160 * 1024 && 8 * 32 * kEpilogueStride * 4 <= kLdsBytes, "LDS budget");
+constexpr int kEpilogueStride = kWaveCols + 8;  // floats per staged row; the padding keeps 16-byte alignment and
+                                                // sends rows 4 apart to different bank halves
+static_assert(kBK == 64 && kLoadsPerStep >= 1 && kLoadsPerStep * (kBK / 16) == kLoadsPerOperand, "pipeline shape");
+static_assert(kLdsBytes <= 160 * 1024 && kWaves * 32 * kEpilogueStride * 4 <= kLdsBytes, "LDS budget");
 
 // ---- LDS layouts ---------------------------------------------------------------------------------------
 // K-contiguous operand, [256 rows][kBK k]: 16-byte chunk c (8 k values) of row r sits at
@@ -97,7 +105,7 @@ __device__ __forceinline__ int lds_offset_row_major(int k, int row) {
 // number (p / 64) % kLoadsPerOperand, so a wavefront writes 1 KiB of consecutive LDS per instruction.
 template <bool kContiguousK>
 struct TileLoader {
-    const char *base;                   // wave-uniform: first row of the tile, first k of the current slice
+    const char *base;                   // wave-uniform: first row of the tile, first k of the loop
     uint32_t offset[kLoadsPerOperand];  // per lane, bytes from `base` (fits 32 bits: checked on the host)
     int64_t step;                       // bytes from one slice to the next
     int lds_offset;                     // of this lane's first slot
@@ -127,18 +135,16 @@ struct TileLoader {
 
     // Buffer loads: scalar base (in the resource descriptor) + 32-bit lane offset, so the addresses cost one
     // register per load and advancing to the next slice is scalar arithmetic.
-    // Load j of the current slice; `advance` moves on to the next slice (after its last load).
-    __device__ __forceinline__ void load_one(u32x4_t (&regs)[kLoadsPerOperand], int j) {
+    // Chunk j of slice `slice` (counted from the first slice of the loop) into regs[j].
+    __device__ __forceinline__ void load_one(u32x4_t (&regs)[kLoadsPerOperand], int j, int slice) {
         const __amdgpu_buffer_rsrc_t resource =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, -1, kBufferResourceFlags);
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base + slice * step), 0, -1, kBufferResourceFlags);
         regs[j] = __builtin_bit_cast(
             u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, static_cast<int>(offset[j]), 0, 0));
     }
-    __device__ __forceinline__ void advance() { base += step; }
-    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand]) {
+    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand], int slice) {
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) load_one(regs, j);
-        advance();
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_one(regs, j, slice);
     }
 
     // Write a landed slice (or its chunk j) into LDS.
@@ -317,18 +323,19 @@ __device__ __forceinline__ const char *uniform_pointer(const char *pointer) {
 // x 64 columns (full 128-byte lines for 2-byte outputs). Row stride 72 floats keeps both the scalar writes (two
 // row groups 4 rows apart per instruction) and the 16-byte reads free of bank conflicts.
 template <typename OutT>
-__device__ __forceinline__ void store_tile(const f32x16_t (&acc)[4][2], FM_LDS(char) * lds, OutT *out, int64_t stride,
+__device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds, OutT *out, int64_t stride,
                                            int rows_valid, int cols_valid, bool accumulate, int wave, int lane) {
-    const int wave_m = wave >> 2, wave_n = wave & 3;
+    constexpr int kLanesPerRow = kWaveCols / 4, kRowsPerStore = 64 / kLanesPerRow;
+    const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
     FM_LDS(float) *staging = reinterpret_cast<FM_LDS(float) *>(lds) + wave * (32 * kEpilogueStride);
-    const int column = (lane & 15) * 4;  // within the wavefront's 64 columns
+    const int column = (lane % kLanesPerRow) * 4;  // within the wavefront's columns
     const int column_in_tile = wave_n * kWaveCols + column;
     // cols_valid is a multiple of 8, so a group of 4 columns is valid or not as a whole.
     const bool column_ok = column_in_tile < cols_valid;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kTilesM; ++i) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v)
                 staging[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * kEpilogueStride + j * 32 + (lane & 31)] =
@@ -337,8 +344,8 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[4][2], FM_LDS(c
         // so no barrier is needed; the empty asm only keeps the compiler from moving accesses across the phases.
         asm volatile("" ::: "memory");
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const int staged_row = t * 4 + (lane >> 4);
+        for (int t = 0; t < 32 / kRowsPerStore; ++t) {
+            const int staged_row = t * kRowsPerStore + lane / kLanesPerRow;
             const int row = wave_m * kWaveRows + i * 32 + staged_row;
             const f32x4_t value = *reinterpret_cast<FM_LDS(f32x4_t) *>(staging + staged_row * kEpilogueStride + column);
             if (row < rows_valid && column_ok) {
@@ -361,7 +368,7 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[4][2], FM_LDS(c
 
 // kMasked: the row-sparse product, whose reduction range [k_lo, k_hi) is ragged.
 template <typename T, bool kLhsContiguousK, bool kRhsContiguousK, bool kMasked>
-__global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(GemmArgs args) {
+__global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_kernel(GemmArgs args) {
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);  // C-style: address-space cast
 
@@ -372,7 +379,7 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wave_m = wave >> 2, wave_n = wave & 3;
+    const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
     // Tile coordinates are the same in every lane; say so, so that they live in scalar registers.
     work.k_lo = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_lo));
     work.k_hi = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_hi));
@@ -395,105 +402,157 @@ __global__ __launch_bounds__(kMfmaThreads, 2) void grouped_gemm_mfma_kernel(Gemm
                        work.cols_valid, wave, lane);
     }
 
-    f32x16_t acc[4][2];
+    f32x16_t acc[kTilesM][kTilesN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kTilesM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // Register sets 0/1 hold the slices in flight; slice s travels in set s % 2 and ends in LDS slot s % 2.
+    // ---- the software pipeline --------------------------------------------------------------------------
+    // Slice s travels through register set s % 2 and ends in LDS slot s % 2. A slice is moved in kBK / 16 chunk
+    // groups (group g = loads g * kLoadsPerStep ..), one group per K-step. During iteration t (multiplying slice t):
+    //   K-steps 0..2 : groups 1..3 of slice t + 1 go registers -> LDS, their registers are refilled from slice t + 3;
+    //   barrier      : slice t + 1 is complete and visible; nobody reads the slot of slice t any more except through
+    //                  fragments already in registers (those of K-step 3 were read during K-step 2);
+    //   K-step 3     : group 0 of slice t + 2 goes to the slot slice t just left, refill from slice t + 4; the
+    //                  fragments of K-step 0 of slice t + 1 are read.
+    // Fragments are double-buffered over K-steps, across slices as well, so the matrix pipe never waits for LDS after
+    // a barrier. The steady-state code has no branch around a load, which lets the compiler guard a register set
+    // with vmcnt(N > 0) instead of draining the queue.
     u32x4_t lhs_regs[2][kLoadsPerOperand], rhs_regs[2][kLoadsPerOperand];
+    u32x4_t frag_a[kTilesM], frag_b[2][kTilesN];
+    constexpr int kSteps = kBK / 16;
     auto stage_of = [&](int slice) { return lds + (slice & 1) * kStageBytes; };
-    auto write_slice = [&](int slice, auto set) {
-        load_lhs.store(lhs_regs[set], stage_of(slice));
-        load_rhs.store(rhs_regs[set], stage_of(slice) + kOperandBytes);
+    // The rhs fragments of a K-step are all in use until its last MFMAs, so they are double-buffered; an lhs fragment
+    // is only used by kTilesN consecutive MFMAs and is re-read for the next K-step right after them.
+    auto read_rhs_fragments = [&](int slice, int kstep, int buffer) {
+#pragma unroll
+        for (int j = 0; j < kTilesN; ++j)
+            frag_b[buffer][j] = load_fragment<kRhsContiguousK>(stage_of(slice) + kOperandBytes,
+                                                               wave_n * kWaveCols + j * 32, kstep, lane);
     };
-    auto fetch_slice = [&](auto set) {
-        load_lhs.load(lhs_regs[set]);
-        load_rhs.load(rhs_regs[set]);
+    auto read_lhs_fragment = [&](int slice, int kstep, int i) {
+        frag_a[i] = load_fragment<kLhsContiguousK>(stage_of(slice), wave_m * kWaveRows + i * 32, kstep, lane);
     };
-    // Multiply slice `slice` from LDS. With `steady`, the traffic for the slices behind it is spread over the four
-    // K-steps instead of being a burst after the barrier: chunk q of slice + 1 goes from register set `set` to LDS
-    // and the freed registers are refilled with chunk q of slice + 3, while the MFMAs of K-step q run.
-    auto multiply_slice = [&](int slice, auto set, auto steady) {
-        FM_LDS(char) *stage = stage_of(slice);
-        FM_LDS(char) *next_stage = stage_of(slice + 1);
+    auto read_fragments = [&](int slice, int kstep, int buffer) {
+        read_rhs_fragments(slice, kstep, buffer);
 #pragma unroll
-        for (int kstep = 0; kstep < kBK / 16; ++kstep) {
-            u32x4_t frag_b[2];
+        for (int i = 0; i < kTilesM; ++i) read_lhs_fragment(slice, kstep, i);
+    };
+    // Chunk group `group` of slice `slice`: registers -> LDS, then refill the registers from slice + 2.
+    auto move_group = [&](int slice, int group, auto set, auto steady) {
+        constexpr bool kSteady = decltype(steady)::value;
+        if (kSteady || slice < num_slices) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                frag_b[j] =
-                    load_fragment<kRhsContiguousK>(stage + kOperandBytes, wave_n * kWaveCols + j * 32, kstep, lane);
-            if constexpr (decltype(steady)::value) {
-                load_lhs.store_one(lhs_regs[set], next_stage, kstep);
-                load_rhs.store_one(rhs_regs[set], next_stage + kOperandBytes, kstep);
-                load_lhs.load_one(lhs_regs[set], kstep);
-                load_rhs.load_one(rhs_regs[set], kstep);
-                if (kstep == kBK / 16 - 1) {
-                    load_lhs.advance();
-                    load_rhs.advance();
-                }
+            for (int q = 0; q < kLoadsPerStep; ++q) {
+                load_lhs.store_one(lhs_regs[set], stage_of(slice), group * kLoadsPerStep + q);
+                load_rhs.store_one(rhs_regs[set], stage_of(slice) + kOperandBytes, group * kLoadsPerStep + q);
             }
+        }
+        if (kSteady || slice + 2 < num_slices) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const u32x4_t frag_a = load_fragment<kLhsContiguousK>(stage, wave_m * kWaveRows + i * 32, kstep, lane);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(frag_a, frag_b[j], acc[i][j]);
+            for (int q = 0; q < kLoadsPerStep; ++q) {
+                load_lhs.load_one(lhs_regs[set], group * kLoadsPerStep + q, slice + 2);
+                load_rhs.load_one(rhs_regs[set], group * kLoadsPerStep + q, slice + 2);
             }
-            // One K-step is one scheduling region: the compiler may interleave inside it but not merge the memory
-            // traffic of several K-steps into one burst.
-            __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // One iteration: after the barrier slice t is visible in LDS slot t % 2 and slot (t + 1) % 2 is free. Slice
-    // t + 1 (in flight for two iterations) goes from its register set to that slot, the set is refilled with
-    // slice t + 3, then slice t is multiplied while t + 2 and t + 3 are in flight.
-    // `steady`: slices t + 1 and t + 3 exist, nothing is conditional. The compiler places the `s_waitcnt vmcnt`
-    // that guards a register set; only where every load on the way is unconditional does it know that 8 newer
-    // loads are outstanding and waits with vmcnt(8..15) instead of draining the queue, so the steady-state loop and
-    // the prologue that leads into it are kept free of branches around loads.
-    auto iteration = [&](int t, auto next_set, auto steady) {
-        __syncthreads();
+    auto mask_slice = [&](int slice) {
         if constexpr (kMasked) {
-            const int k0 = static_cast<int>(k_first) + t * kBK;
-            if (k0 < work.k_lo || k0 + kBK > work.k_hi) {  // wave-uniform: first/last slice of the range
-                mask_tile<kLhsContiguousK>(stage_of(t), k0, work.k_lo, work.k_hi);
-                mask_tile<kRhsContiguousK>(stage_of(t) + kOperandBytes, k0, work.k_lo, work.k_hi);
+            const int k0 = static_cast<int>(k_first) + slice * kBK;
+            if (slice < num_slices && (k0 < work.k_lo || k0 + kBK > work.k_hi)) {  // wave-uniform
+                mask_tile<kLhsContiguousK>(stage_of(slice), k0, work.k_lo, work.k_hi);
+                mask_tile<kRhsContiguousK>(stage_of(slice) + kOperandBytes, k0, work.k_lo, work.k_hi);
                 __syncthreads();
             }
         }
-        if constexpr (decltype(steady)::value) {
-            multiply_slice(t, next_set, std::true_type{});
-        } else {
-            if (t + 1 < num_slices) write_slice(t + 1, next_set);
-            if (t + 3 < num_slices) fetch_slice(next_set);
-            multiply_slice(t, next_set, std::false_type{});
+    };
+    // `next_set` holds slice t + 1, `other_set` slice t + 2.
+    auto iteration = [&](int t, auto next_set, auto other_set, auto steady) {
+        constexpr bool kSteady = decltype(steady)::value;
+#pragma unroll
+        for (int kstep = 0; kstep < kSteps; ++kstep) {
+            const bool has_next = kSteady || kstep + 1 < kSteps || t + 1 < num_slices;
+            const int next_slice = kstep + 1 < kSteps ? t : t + 1, next_kstep = (kstep + 1) % kSteps;
+            if (has_next) read_rhs_fragments(next_slice, next_kstep, (kstep + 1) & 1);
+            if (kstep + 1 < kSteps) move_group(t + 1, kstep + 1, next_set, steady);
+            else move_group(t + 2, 0, other_set, steady);
+#pragma unroll
+            for (int i = 0; i < kTilesM; ++i) {
+#pragma unroll
+                for (int j = 0; j < kTilesN; ++j) acc[i][j] = Mfma<T>::run(frag_a[i], frag_b[kstep & 1][j], acc[i][j]);
+                if (has_next) read_lhs_fragment(next_slice, next_kstep, i);
+            }
+            // One K-step is one scheduling region. Inside it, ask for one memory instruction in the shadow of every
+            // MFMA (an MFMA keeps the matrix pipe busy for 32 cycles, a clump of LDS/global instructions longer than
+            // that leaves it idle): fragment reads first, then the LDS writes, then the global loads.
+            if constexpr (kSteady) {
+                // Memory instructions of a K-step in program order: kTilesN rhs fragment reads, 2 kLoadsPerStep LDS
+                // writes, 2 kLoadsPerStep global loads, and one lhs fragment read after each group of kTilesN MFMAs.
+                constexpr int kOthers = kTilesN + 4 * kLoadsPerStep;  // besides the lhs reads
+#pragma unroll
+                for (int m = 0; m < kTilesM * kTilesN; ++m) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                    if ((m + 1) % kTilesN == 0) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // lhs fragment read
+                    } else {
+                        // spread the other memory instructions over the remaining MFMA shadows
+                        constexpr int kSlots = kTilesM * (kTilesN - 1);
+                        const int slot = m - m / kTilesN;  // index among the MFMAs that do not end a group
+                        const int first = slot * kOthers / kSlots, last = (slot + 1) * kOthers / kSlots;
+                        for (int o = first; o < last; ++o) {
+                            if (o < kTilesN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                            else if (o < kTilesN + 2 * kLoadsPerStep) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                            else __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        }
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (kstep == kSteps - 2) {
+                __syncthreads();
+                mask_slice(t + 1);
+            }
         }
     };
     constexpr std::integral_constant<int, 0> set0{};
     constexpr std::integral_constant<int, 1> set1{};
+    auto fetch_slice = [&](int slice, auto set) {
+        load_lhs.load(lhs_regs[set], slice);
+        load_rhs.load(rhs_regs[set], slice);
+    };
+    // Prologue: slice 0 completely into LDS, group 0 of slice 1 as well, slices 1..3 (partly) in flight.
     int t = 0;
-    if (num_slices >= 5) {
-        fetch_slice(set0);
-        fetch_slice(set1);
-        write_slice(0, set0);
-        fetch_slice(set0);
-        for (; t + 4 < num_slices; t += 2) {  // slices up to t + 4 exist
-            iteration(t, set1, std::true_type{});
-            iteration(t + 1, set0, std::true_type{});
+    if (num_slices >= 6) {
+        fetch_slice(0, set0);
+        fetch_slice(1, set1);
+        load_lhs.store(lhs_regs[set0], stage_of(0));
+        load_rhs.store(rhs_regs[set0], stage_of(0) + kOperandBytes);
+        fetch_slice(2, set0);
+        move_group(1, 0, set1, std::true_type{});
+        __syncthreads();
+        mask_slice(0);
+        read_fragments(0, 0, 0);
+        for (; t + 5 < num_slices; t += 2) {  // slices up to t + 5 exist
+            iteration(t, set1, set0, std::true_type{});
+            iteration(t + 1, set0, set1, std::true_type{});
         }
-    } else {
-        if (num_slices > 0) fetch_slice(set0);
-        if (num_slices > 1) fetch_slice(set1);
-        if (num_slices > 0) write_slice(0, set0);
-        if (num_slices > 2) fetch_slice(set0);
+    } else if (num_slices > 0) {
+        fetch_slice(0, set0);
+        if (num_slices > 1) fetch_slice(1, set1);
+        load_lhs.store(lhs_regs[set0], stage_of(0));
+        load_rhs.store(rhs_regs[set0], stage_of(0) + kOperandBytes);
+        if (num_slices > 2) fetch_slice(2, set0);
+        move_group(1, 0, set1, std::false_type{});
+        __syncthreads();
+        mask_slice(0);
+        read_fragments(0, 0, 0);
     }
-    for (; t < num_slices; t += 2) {  // the last (at most four) slices
-        iteration(t, set1, std::false_type{});
-        if (t + 1 < num_slices) iteration(t + 1, set0, std::false_type{});
+    for (; t < num_slices; t += 2) {  // the last slices: same schedule, every transfer conditional
+        iteration(t, set1, set0, std::false_type{});
+        if (t + 1 < num_slices) iteration(t + 1, set0, set1, std::false_type{});
     }
 
     const bool accumulate = args.accumulate != 0;
