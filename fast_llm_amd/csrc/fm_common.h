@@ -75,6 +75,18 @@ __device__ __forceinline__ void store16(T *pointer, const Vec16<T> &value) {
     *reinterpret_cast<Vec16<T> *>(pointer) = value;
 }
 
+// Streaming variants: the data is touched once by this kernel and is larger than the caches.
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t RawVec16;
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16_stream(const T *pointer) {
+    const RawVec16 raw = __builtin_nontemporal_load(reinterpret_cast<const RawVec16 *>(pointer));
+    return __builtin_bit_cast(Vec16<T>, raw);
+}
+template <typename T>
+__device__ __forceinline__ void store16_stream(T *pointer, const Vec16<T> &value) {
+    __builtin_nontemporal_store(__builtin_bit_cast(RawVec16, value), reinterpret_cast<RawVec16 *>(pointer));
+}
+
 __device__ __forceinline__ float wave_sum(float value) {
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) value += __shfl_xor(value, offset, 64);

@@ -141,7 +141,7 @@ __global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__res
                     Vec16<T> scaled;
 #pragma unroll
                     for (int i = 0; i < N; ++i) scaled.v[i] = from_float<T>(to_float(g.v[i]) * score);
-                    if constexpr (kVector) store16(out_row + c, scaled);
+                    if constexpr (kVector) store16_stream(out_row + c, scaled);
                     else out_row[c] = scaled.v[0];
                 }
             };
