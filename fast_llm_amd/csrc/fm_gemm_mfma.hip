@@ -45,6 +45,13 @@ struct alignas(4 * sizeof(T)) Vec16x4 {
     T v[4];
 };
 
+// The output tile is written once and not read again by this kernel: keep it from displacing operand panels in L2.
+template <typename T>
+__device__ __forceinline__ void store_streaming(T *pointer, const Vec16x4<T> &value) {
+    typedef __attribute__((__vector_size__(4 * sizeof(T)))) std::conditional_t<sizeof(T) == 4, uint32_t, uint16_t> Raw;
+    __builtin_nontemporal_store(__builtin_bit_cast(Raw, value), reinterpret_cast<Raw *>(pointer));
+}
+
 #define FM_LDS(T) __attribute__((address_space(3))) T
 #define FM_GLOBAL(T) __attribute__((address_space(1))) T
 
@@ -71,8 +78,7 @@ constexpr int kWaves = kWavesM * kWavesN, kMfmaThreads = 64 * kWaves;
 constexpr int kBK = 64;      // K elements per slice (32 or 64)
 constexpr int kStages = 2;   // LDS slots
 constexpr int kOperandBytes = kTile * kBK * 2;  // one operand slice in LDS, same size in either layout
-constexpr int kStageBytes = 2 * kOperandBytes;  // lhs slice, then rhs slice
-constexpr int kLdsBytes = kStages * kStageBytes;
+constexpr int kLdsBytes = 2 * kStages * kOperandBytes;  // the lhs slots, then the rhs slots
 constexpr int kWaveRows = kTile / kWavesM, kWaveCols = kTile / kWavesN;  // a wavefront's part of the tile
 constexpr int kTilesM = kWaveRows / 32, kTilesN = kWaveCols / 32;        // in 32x32 MFMA accumulators
 constexpr int kChunksPerRow = kBK / 8;          // 16-byte chunks of a K-major row
@@ -100,28 +106,44 @@ __device__ __forceinline__ int lds_offset_row_major(int k, int row) {
     return k * (kTile * 2) + ((((row >> 4) ^ ((k & 3) << 1)) << 5) | ((row & 15) << 1));
 }
 
+// Tell the compiler that a pointer computed from tile coordinates is the same in every lane (it then lives in
+// scalar registers and the loads use the scalar-base addressing form).
+__device__ __forceinline__ const char *uniform_pointer(const char *pointer) {
+    const uint64_t bits = reinterpret_cast<uint64_t>(pointer);
+    const uint32_t low = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+    const uint32_t high = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+    return reinterpret_cast<const char *>((static_cast<uint64_t>(high) << 32) | low);
+}
+
 // Loader of one operand slice: global memory -> registers -> LDS. The slice is 256 * kBK / 8 chunks of 16 bytes;
 // chunk slot p of the LDS slice is handled by lane p % 64 of wavefront (p / 64) / kLoadsPerOperand as its load
 // number (p / 64) % kLoadsPerOperand, so a wavefront writes 1 KiB of consecutive LDS per instruction.
 template <bool kContiguousK>
 struct TileLoader {
-    const char *base;                   // wave-uniform: first row of the tile, first k of the loop
-    uint32_t offset[kLoadsPerOperand];  // per lane, bytes from `base` (fits 32 bits: checked on the host)
-    int64_t step;                       // bytes from one slice to the next
-    int lds_offset;                     // of this lane's first slot
+    const char *fetch_base;  // wave-uniform: first row of the tile, first k of the slice being fetched
+    uint32_t offset[2];      // per lane, bytes from `fetch_base`, of loads 0 and 1 (fits 32 bits: checked on the host)
+    uint32_t pair_stride;    // wave-uniform: bytes from load j to load j + 2 (the swizzles repeat with period 2)
+    uint32_t num_records;    // wave-uniform: lane offsets >= this read as zero
+    int64_t step;            // bytes from one slice to the next
+    int slices_left;         // slices after the one being fetched
+    int lds_offset;          // of this lane's first slot
 
-    // `stride`: bytes between rows (K-contiguous) or between K-rows (row-contiguous). Rows >= valid_rows are
-    // replaced by in-range ones (their products are never stored).
-    __device__ __forceinline__ void setup(const char *tile_base, int64_t stride, int valid_rows, int wave, int lane) {
-        base = tile_base;
+    // `stride`: bytes between rows (K-contiguous) or between K-rows (row-contiguous). Rows >= valid_rows are never
+    // stored; a K-contiguous operand reads them as zero (they lie past the range of the buffer descriptor), a
+    // row-contiguous one reads in-range rows in their place.
+    __device__ __forceinline__ void setup(const char *tile_base, int64_t stride, int valid_rows, int num_slices,
+                                          int wave, int lane) {
+        static_assert(kLoadsPerOperand % 2 == 0, "loads come in (even, odd) pairs");
+        fetch_base = tile_base;
+        slices_left = num_slices - 1;
         lds_offset = (wave * kLoadsPerOperand * 64 + lane) * 16;
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) {
+        for (int j = 0; j < 2; ++j) {
             const int slot = (wave * kLoadsPerOperand + j) * 64 + lane;
             if constexpr (kContiguousK) {
                 const int row = slot / kChunksPerRow;
                 const int chunk = (slot % kChunksPerRow) ^ k_major_swizzle(row);
-                offset[j] = static_cast<uint32_t>(min(row, valid_rows - 1) * stride + chunk * 16);
+                offset[j] = static_cast<uint32_t>(row * stride + chunk * 16);
             } else {
                 const int k = slot >> 5, position = slot & 31;
                 const int group = (position >> 1) ^ ((k & 3) << 1);
@@ -130,21 +152,35 @@ struct TileLoader {
                 offset[j] = static_cast<uint32_t>(k * stride + first_row * 2);
             }
         }
+        // Two loads further on: 128 slots = 16 rows of a K-contiguous slice, 4 K-rows of a row-contiguous one.
+        pair_stride = static_cast<uint32_t>((kContiguousK ? 128 / kChunksPerRow : 4) * stride);
+        num_records = kContiguousK ? static_cast<uint32_t>((valid_rows - 1) * stride + kBK * 2) : 0xffffffffu;
         step = kContiguousK ? kBK * 2 : kBK * stride;
     }
 
-    // Buffer loads: scalar base (in the resource descriptor) + 32-bit lane offset, so the addresses cost one
-    // register per load and advancing to the next slice is scalar arithmetic.
-    // Chunk j of slice `slice` (counted from the first slice of the loop) into regs[j].
-    __device__ __forceinline__ void load_one(u32x4_t (&regs)[kLoadsPerOperand], int j, int slice) {
-        const __amdgpu_buffer_rsrc_t resource =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base + slice * step), 0, -1, kBufferResourceFlags);
-        regs[j] = __builtin_bit_cast(
-            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, static_cast<int>(offset[j]), 0, 0));
+    // Move on to the next slice. Past the last slice the descriptor's range becomes empty, so that every further
+    // load brings zeros without touching memory: the pipeline can run a slice too far without a branch.
+    __device__ __forceinline__ void advance() {
+        // Said to be wave-uniform once more: loop-carried values otherwise end up in vector registers.
+        fetch_base = uniform_pointer(fetch_base + step);
+        slices_left = __builtin_amdgcn_readfirstlane(slices_left - 1);
+        num_records = __builtin_amdgcn_readfirstlane(slices_left < 0 ? 0u : num_records);
     }
-    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand], int slice) {
+
+    // Buffer loads: scalar base (in the resource descriptor) + 32-bit lane offset, so the addresses cost two
+    // registers per operand and advancing to the next slice is scalar arithmetic.
+    // Chunk j of the slice being fetched into regs[j].
+    __device__ __forceinline__ void load_one(u32x4_t (&regs)[kLoadsPerOperand], int j) {
+        const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char *>(uniform_pointer(fetch_base)), 0,
+            static_cast<int>(__builtin_amdgcn_readfirstlane(num_records)), kBufferResourceFlags);
+        const uint32_t lane_offset = offset[j & 1] + static_cast<uint32_t>(j >> 1) * pair_stride;
+        regs[j] = __builtin_bit_cast(
+            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, static_cast<int>(lane_offset), 0, 0));
+    }
+    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand]) {
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) load_one(regs, j, slice);
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_one(regs, j);
     }
 
     // Write a landed slice (or its chunk j) into LDS.
@@ -158,23 +194,34 @@ struct TileLoader {
     }
 };
 
-// MFMA operand fragment (8 consecutive k of one row per lane; lane l: row l % 32, k half l / 32) of the 32 rows
-// starting at `row_base`, for the 16-wide K slice `kstep` of the tile.
+// MFMA operand fragments (8 consecutive k of one row per lane; lane l: row l % 32, k half l / 32). A wavefront reads
+// 4 fragments (32 rows each, `i`) for each of the 4 K-steps of a slice, from either LDS slot. Thanks to the period of
+// the swizzles, 4 per-lane addresses per operand are enough; everything else is an immediate offset of the LDS
+// instruction: a K-contiguous operand needs one address per K-step (fragment i is 32 rows = 4 KiB further on), a
+// row-contiguous one needs one per fragment (K-step s is 16 K-rows = 8 KiB further on).
 template <bool kContiguousK>
-__device__ __forceinline__ u32x4_t load_fragment(FM_LDS(char) * operand_lds, int row_base, int kstep, int lane) {
+__device__ __forceinline__ int fragment_base(int row_base, int q, int lane) {
     if constexpr (kContiguousK) {
-        const int offset = lds_offset_k_major(row_base + (lane & 31), kstep * 2 + (lane >> 5));
-        return *reinterpret_cast<FM_LDS(u32x4_t) *>(operand_lds + offset);
+        return lds_offset_k_major(row_base + (lane & 31), q * 2 + (lane >> 5));
     } else {
         // ds_read_b64_tr_b16 works on groups of 16 lanes: lane s of a group supplies the address of 4 rows
         // (row0 + 4 (s % 4) ..) at K-row k0 + s / 4 and receives k0 .. k0 + 3 of row row0 + s.
         const int s = lane & 15, group = lane >> 4;
-        const int row = row_base + ((group & 1) << 4) + ((s & 3) << 2);
-        const int k = kstep * 16 + ((group >> 1) << 3) + (s >> 2);
-        const i16x4_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            reinterpret_cast<FM_LDS(i16x4_t) *>(operand_lds + lds_offset_row_major(k, row)));
-        const i16x4_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            reinterpret_cast<FM_LDS(i16x4_t) *>(operand_lds + lds_offset_row_major(k + 4, row)));
+        const int row = row_base + q * 32 + ((group & 1) << 4) + ((s & 3) << 2);
+        const int k = ((group >> 1) << 3) + (s >> 2);
+        return lds_offset_row_major(k, row);
+    }
+}
+// `bases`: fragment_base of q = 0..3 plus the LDS offset of the operand's slot 0.
+template <bool kContiguousK>
+__device__ __forceinline__ u32x4_t load_fragment(FM_LDS(char) * lds, const int (&bases)[4], int slot, int i, int kstep) {
+    if constexpr (kContiguousK) {
+        return *reinterpret_cast<FM_LDS(u32x4_t) *>(lds + bases[kstep] + (slot * kOperandBytes + i * 32 * kBK * 2));
+    } else {
+        FM_LDS(char) *address = lds + bases[i] + (slot * kOperandBytes + kstep * 16 * kTile * 2);
+        const i16x4_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<FM_LDS(i16x4_t) *>(address));
+        const i16x4_t high =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<FM_LDS(i16x4_t) *>(address + 4 * kTile * 2));
         const u32x2_t low_words = __builtin_bit_cast(u32x2_t, low), high_words = __builtin_bit_cast(u32x2_t, high);
         return u32x4_t{low_words[0], low_words[1], high_words[0], high_words[1]};
     }
@@ -309,15 +356,6 @@ __device__ __forceinline__ void tile_of_block(const GemmArgs &args, int &tile_m,
 }
 
 // ---- the kernel ----------------------------------------------------------------------------------------
-// Tell the compiler that a pointer computed from tile coordinates is the same in every lane (it then lives in
-// scalar registers and the loads use the scalar-base addressing form).
-__device__ __forceinline__ const char *uniform_pointer(const char *pointer) {
-    const uint64_t bits = reinterpret_cast<uint64_t>(pointer);
-    const uint32_t low = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
-    const uint32_t high = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
-    return reinterpret_cast<const char *>((static_cast<uint64_t>(high) << 32) | low);
-}
-
 // Write the wavefront's 128 x 64 accumulators through its own LDS region, 32 rows at a time: registers -> LDS as
 // [32][kEpilogueStride] floats, then every lane takes 4 consecutive columns, so one store instruction covers 4 rows
 // x 64 columns (full 128-byte lines for 2-byte outputs). Row stride 72 floats keeps both the scalar writes (two
@@ -359,7 +397,7 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTiles
 #pragma unroll
                     for (int c = 0; c < 4; ++c) packed.v[c] = from_float<OutT>(value[c]);
                 }
-                *reinterpret_cast<Vec16x4<OutT> *>(pointer) = packed;
+                store_streaming(pointer, packed);
             }
         }
         asm volatile("" ::: "memory");
@@ -397,9 +435,9 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         const char *rhs = static_cast<const char *>(args.rhs) +
                           (work.rhs_offset + k_first * args.rhs_stride_inner) * static_cast<int64_t>(sizeof(T));
         load_lhs.setup(uniform_pointer(lhs), (kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner) * sizeof(T),
-                       work.rows_valid, wave, lane);
+                       work.rows_valid, num_slices, wave, lane);
         load_rhs.setup(uniform_pointer(rhs), (kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner) * sizeof(T),
-                       work.cols_valid, wave, lane);
+                       work.cols_valid, num_slices, wave, lane);
     }
 
     f32x16_t acc[kTilesM][kTilesN];
@@ -418,141 +456,131 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     //                  fragments already in registers (those of K-step 3 were read during K-step 2);
     //   K-step 3     : group 0 of slice t + 2 goes to the slot slice t just left, refill from slice t + 4; the
     //                  fragments of K-step 0 of slice t + 1 are read.
-    // Fragments are double-buffered over K-steps, across slices as well, so the matrix pipe never waits for LDS after
-    // a barrier. The steady-state code has no branch around a load, which lets the compiler guard a register set
-    // with vmcnt(N > 0) instead of draining the queue.
+    // The pipeline has no branch around a transfer, which lets the compiler guard a register set with vmcnt(N > 0)
+    // instead of draining the queue: loads past the last slice bring zeros.
     u32x4_t lhs_regs[2][kLoadsPerOperand], rhs_regs[2][kLoadsPerOperand];
     u32x4_t frag_a[kTilesM], frag_b[2][kTilesN];
     constexpr int kSteps = kBK / 16;
-    auto stage_of = [&](int slice) { return lds + (slice & 1) * kStageBytes; };
+    // Slice s sits in slot s % 2 of either operand. Slots are passed around as compile-time constants so that they
+    // end up in the immediate offsets of the LDS instructions.
+    auto lhs_slot = [&](int slot) { return lds + slot * kOperandBytes; };
+    auto rhs_slot = [&](int slot) { return lds + (kStages + slot) * kOperandBytes; };
+    int lhs_frag[4], rhs_frag[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        lhs_frag[q] = fragment_base<kLhsContiguousK>(wave_m * kWaveRows, q, lane);
+        rhs_frag[q] = kStages * kOperandBytes + fragment_base<kRhsContiguousK>(wave_n * kWaveCols, q, lane);
+    }
     // The rhs fragments of a K-step are all in use until its last MFMAs, so they are double-buffered; an lhs fragment
     // is only used by kTilesN consecutive MFMAs and is re-read for the next K-step right after them.
-    auto read_rhs_fragments = [&](int slice, int kstep, int buffer) {
-#pragma unroll
-        for (int j = 0; j < kTilesN; ++j)
-            frag_b[buffer][j] = load_fragment<kRhsContiguousK>(stage_of(slice) + kOperandBytes,
-                                                               wave_n * kWaveCols + j * 32, kstep, lane);
+    auto read_rhs_fragment = [&](int slot, int kstep, int buffer, int j) {
+        frag_b[buffer][j] = load_fragment<kRhsContiguousK>(lds, rhs_frag, slot, j, kstep);
     };
-    auto read_lhs_fragment = [&](int slice, int kstep, int i) {
-        frag_a[i] = load_fragment<kLhsContiguousK>(stage_of(slice), wave_m * kWaveRows + i * 32, kstep, lane);
+    auto read_lhs_fragment = [&](int slot, int kstep, int i) {
+        frag_a[i] = load_fragment<kLhsContiguousK>(lds, lhs_frag, slot, i, kstep);
     };
-    auto read_fragments = [&](int slice, int kstep, int buffer) {
-        read_rhs_fragments(slice, kstep, buffer);
+    auto read_fragments = [&](int slot, int kstep, int buffer) {
 #pragma unroll
-        for (int i = 0; i < kTilesM; ++i) read_lhs_fragment(slice, kstep, i);
+        for (int j = 0; j < kTilesN; ++j) read_rhs_fragment(slot, kstep, buffer, j);
+#pragma unroll
+        for (int i = 0; i < kTilesM; ++i) read_lhs_fragment(slot, kstep, i);
     };
-    // Chunk group `group` of slice `slice`: registers -> LDS, then refill the registers from slice + 2.
-    auto move_group = [&](int slice, int group, auto set, auto steady) {
-        constexpr bool kSteady = decltype(steady)::value;
-        if (kSteady || slice < num_slices) {
-#pragma unroll
-            for (int q = 0; q < kLoadsPerStep; ++q) {
-                load_lhs.store_one(lhs_regs[set], stage_of(slice), group * kLoadsPerStep + q);
-                load_rhs.store_one(rhs_regs[set], stage_of(slice) + kOperandBytes, group * kLoadsPerStep + q);
-            }
-        }
-        if (kSteady || slice + 2 < num_slices) {
-#pragma unroll
-            for (int q = 0; q < kLoadsPerStep; ++q) {
-                load_lhs.load_one(lhs_regs[set], group * kLoadsPerStep + q, slice + 2);
-                load_rhs.load_one(rhs_regs[set], group * kLoadsPerStep + q, slice + 2);
-            }
-        }
-    };
-    auto mask_slice = [&](int slice) {
+    auto mask_slice = [&](int slice, int slot) {
         if constexpr (kMasked) {
             const int k0 = static_cast<int>(k_first) + slice * kBK;
             if (slice < num_slices && (k0 < work.k_lo || k0 + kBK > work.k_hi)) {  // wave-uniform
-                mask_tile<kLhsContiguousK>(stage_of(slice), k0, work.k_lo, work.k_hi);
-                mask_tile<kRhsContiguousK>(stage_of(slice) + kOperandBytes, k0, work.k_lo, work.k_hi);
+                mask_tile<kLhsContiguousK>(lhs_slot(slot), k0, work.k_lo, work.k_hi);
+                mask_tile<kRhsContiguousK>(rhs_slot(slot), k0, work.k_lo, work.k_hi);
                 __syncthreads();
             }
         }
     };
     // `next_set` holds slice t + 1, `other_set` slice t + 2.
-    auto iteration = [&](int t, auto next_set, auto other_set, auto steady) {
-        constexpr bool kSteady = decltype(steady)::value;
+    // A K-step is 16 slots of "one MFMA, then one memory instruction in its shadow" (an MFMA keeps the matrix pipe busy
+    // for 32 cycles; a clump of LDS/global instructions longer than that leaves it idle). The order is pinned with a
+    // scheduling barrier after every slot, because what a fragment read may overtake decides how long before its use
+    // it is issued: left to itself the scheduler reads the lhs fragment of the first MFMAs of a K-step last.
+    //   slots 0..3       rhs fragments 0..3 of the next K-step (other fragment buffer)
+    //   slots 4, 8, 12   lhs fragments 0, 1, 2 of the next K-step, each right after the last MFMA of its predecessor
+    //   slots 5, 6, 9, 10        registers -> LDS (lhs, rhs of chunk 0, then of chunk 1 of the group)
+    //   slots 7, 11, 13, 14      refill of the same registers from two slices further on, in the order of their use
+    //   slot 15          lhs fragment 3 of the next K-step
+    // so every fragment is issued at least 12 MFMAs before its first use.
+    static_assert(kTilesM == 4 && kTilesN == 4 && kLoadsPerStep == 2, "the slot table below is written for this shape");
+    auto iteration = [&](int t, auto next_set, auto other_set) {
+        constexpr int kSlot = decltype(other_set)::value, kNextSlot = decltype(next_set)::value;  // of slices t, t + 1
 #pragma unroll
         for (int kstep = 0; kstep < kSteps; ++kstep) {
-            const bool has_next = kSteady || kstep + 1 < kSteps || t + 1 < num_slices;
-            const int next_slice = kstep + 1 < kSteps ? t : t + 1, next_kstep = (kstep + 1) % kSteps;
-            if (has_next) read_rhs_fragments(next_slice, next_kstep, (kstep + 1) & 1);
-            if (kstep + 1 < kSteps) move_group(t + 1, kstep + 1, next_set, steady);
-            else move_group(t + 2, 0, other_set, steady);
-#pragma unroll
-            for (int i = 0; i < kTilesM; ++i) {
-#pragma unroll
-                for (int j = 0; j < kTilesN; ++j) acc[i][j] = Mfma<T>::run(frag_a[i], frag_b[kstep & 1][j], acc[i][j]);
-                if (has_next) read_lhs_fragment(next_slice, next_kstep, i);
+            const int next_slot = kstep + 1 < kSteps ? kSlot : kNextSlot, next_kstep = (kstep + 1) % kSteps;
+            // The chunk group that moves during this K-step: groups 1..3 of slice t + 1 (refilled from slice t + 3),
+            // then group 0 of slice t + 2 (refilled from slice t + 4).
+            const int group = (kstep + 1) % kSteps;
+            const int set = kstep + 1 < kSteps ? kNextSlot : kSlot, moved_slot = set;
+            if (kstep == kSteps - 1) {
+                load_lhs.advance();
+                load_rhs.advance();
             }
-            // One K-step is one scheduling region. Inside it, ask for one memory instruction in the shadow of every
-            // MFMA (an MFMA keeps the matrix pipe busy for 32 cycles, a clump of LDS/global instructions longer than
-            // that leaves it idle): fragment reads first, then the LDS writes, then the global loads.
-            if constexpr (kSteady) {
-                // Memory instructions of a K-step in program order: kTilesN rhs fragment reads, 2 kLoadsPerStep LDS
-                // writes, 2 kLoadsPerStep global loads, and one lhs fragment read after each group of kTilesN MFMAs.
-                constexpr int kOthers = kTilesN + 4 * kLoadsPerStep;  // besides the lhs reads
 #pragma unroll
-                for (int m = 0; m < kTilesM * kTilesN; ++m) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-                    if ((m + 1) % kTilesN == 0) {
-                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // lhs fragment read
-                    } else {
-                        // spread the other memory instructions over the remaining MFMA shadows
-                        constexpr int kSlots = kTilesM * (kTilesN - 1);
-                        const int slot = m - m / kTilesN;  // index among the MFMAs that do not end a group
-                        const int first = slot * kOthers / kSlots, last = (slot + 1) * kOthers / kSlots;
-                        for (int o = first; o < last; ++o) {
-                            if (o < kTilesN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                            else if (o < kTilesN + 2 * kLoadsPerStep) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                            else __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                        }
-                    }
+            for (int m = 0; m < kTilesM * kTilesN; ++m) {
+                const int i = m / kTilesN, j = m % kTilesN;
+                acc[i][j] = Mfma<T>::run(frag_a[i], frag_b[kstep & 1][j], acc[i][j]);
+                if (m < kTilesN) {
+                    read_rhs_fragment(next_slot, next_kstep, (kstep + 1) & 1, m);
+                } else if (j == 0 || m == kTilesM * kTilesN - 1) {
+                    read_lhs_fragment(next_slot, next_kstep, j == 0 ? i - 1 : i);
+                } else if (m == 5 || m == 9) {
+                    load_lhs.store_one(lhs_regs[set], lhs_slot(moved_slot), group * kLoadsPerStep + m / 8);
+                } else if (m == 6 || m == 10) {
+                    load_rhs.store_one(rhs_regs[set], rhs_slot(moved_slot), group * kLoadsPerStep + m / 8);
+                } else if (m == 7 || m == 13) {
+                    load_lhs.load_one(lhs_regs[set], group * kLoadsPerStep + m / 8);
+                } else {  // 11, 14
+                    load_rhs.load_one(rhs_regs[set], group * kLoadsPerStep + m / 12);
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
             if (kstep == kSteps - 2) {
                 __syncthreads();
-                mask_slice(t + 1);
+                mask_slice(t + 1, kNextSlot);
             }
         }
     };
-    constexpr std::integral_constant<int, 0> set0{};
-    constexpr std::integral_constant<int, 1> set1{};
-    auto fetch_slice = [&](int slice, auto set) {
-        load_lhs.load(lhs_regs[set], slice);
-        load_rhs.load(rhs_regs[set], slice);
-    };
-    // Prologue: slice 0 completely into LDS, group 0 of slice 1 as well, slices 1..3 (partly) in flight.
-    int t = 0;
-    if (num_slices >= 6) {
-        fetch_slice(0, set0);
-        fetch_slice(1, set1);
-        load_lhs.store(lhs_regs[set0], stage_of(0));
-        load_rhs.store(rhs_regs[set0], stage_of(0) + kOperandBytes);
-        fetch_slice(2, set0);
-        move_group(1, 0, set1, std::true_type{});
-        __syncthreads();
-        mask_slice(0);
-        read_fragments(0, 0, 0);
-        for (; t + 5 < num_slices; t += 2) {  // slices up to t + 5 exist
-            iteration(t, set1, set0, std::true_type{});
-            iteration(t + 1, set0, set1, std::true_type{});
+    if (num_slices > 0) {
+        // Prologue: slice 0 completely into LDS, group 0 of slice 1 as well, slices 1..3 (partly) in flight.
+        load_lhs.load(lhs_regs[0]);
+        load_rhs.load(rhs_regs[0]);
+        load_lhs.advance();
+        load_rhs.advance();
+        load_lhs.load(lhs_regs[1]);
+        load_rhs.load(rhs_regs[1]);
+        load_lhs.advance();
+        load_rhs.advance();
+        load_lhs.store(lhs_regs[0], lhs_slot(0));
+        load_rhs.store(rhs_regs[0], rhs_slot(0));
+        load_lhs.load(lhs_regs[0]);
+        load_rhs.load(rhs_regs[0]);
+        load_lhs.advance();
+        load_rhs.advance();
+#pragma unroll
+        for (int q = 0; q < kLoadsPerStep; ++q) {
+            load_lhs.store_one(lhs_regs[1], lhs_slot(1), q);
+            load_rhs.store_one(rhs_regs[1], rhs_slot(1), q);
         }
-    } else if (num_slices > 0) {
-        fetch_slice(0, set0);
-        if (num_slices > 1) fetch_slice(1, set1);
-        load_lhs.store(lhs_regs[set0], stage_of(0));
-        load_rhs.store(rhs_regs[set0], stage_of(0) + kOperandBytes);
-        if (num_slices > 2) fetch_slice(2, set0);
-        move_group(1, 0, set1, std::false_type{});
+#pragma unroll
+        for (int q = 0; q < kLoadsPerStep; ++q) {
+            load_lhs.load_one(lhs_regs[1], q);
+            load_rhs.load_one(rhs_regs[1], q);
+        }
         __syncthreads();
-        mask_slice(0);
+        mask_slice(0, 0);
         read_fragments(0, 0, 0);
-    }
-    for (; t < num_slices; t += 2) {  // the last slices: same schedule, every transfer conditional
-        iteration(t, set1, set0, std::false_type{});
-        if (t + 1 < num_slices) iteration(t + 1, set0, set1, std::false_type{});
+        constexpr std::integral_constant<int, 0> set0{};
+        constexpr std::integral_constant<int, 1> set1{};
+        // Two slices per trip (the register sets and LDS slots alternate); an odd count multiplies one slice of zeros.
+        for (int t = 0; t < num_slices; t += 2) {
+            iteration(t, set1, set0);
+            iteration(t + 1, set0, set1);
+        }
     }
 
     const bool accumulate = args.accumulate != 0;
