@@ -44,7 +44,7 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--warmup", type=int, default=3)
     parser.add_argument("--workload", default="mixtral", help="tiny | mixtral | fine_grained | wide | imbalanced")
     parser.add_argument("--recompute", default="none", help="none | activation | activation_and_input | full")
-    parser.add_argument("--cpu-tokens", type=int, default=4096, help="tokens in the CPU baseline sample (0: skip)")
+    parser.add_argument("--cpu-tokens", type=int, default=8192, help="tokens in the CPU baseline sample (0: skip)")
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument(
         "--calibration-mib",

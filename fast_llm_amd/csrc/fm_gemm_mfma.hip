@@ -85,10 +85,10 @@ constexpr int kChunksPerRow = kBK / 8;          // 16-byte chunks of a K-major r
 constexpr int kLoadsPerOperand = kOperandBytes / 16 / kMfmaThreads;  // 16-byte loads per lane, operand and slice
 constexpr int kLoadsPerStep = kLoadsPerOperand / (kBK / 16);        // of them moved during one K-step
 constexpr int kBufferResourceFlags = 0x00020000;  // raw buffer, 32-bit data format, no swizzle
-constexpr int kEpilogueStride = kWaveCols + 8;  // floats per staged row; the padding keeps 16-byte alignment and
-                                                // sends rows 4 apart to different bank halves
+constexpr int kEpiloguePadBytes = 16;  // after each staged row of the epilogue; keeps 16-byte alignment and spreads
+                                       // the rows over the banks
 static_assert(kBK == 64 && kLoadsPerStep >= 1 && kLoadsPerStep * (kBK / 16) == kLoadsPerOperand, "pipeline shape");
-static_assert(kLdsBytes <= 160 * 1024 && kWaves * 32 * kEpilogueStride * 4 <= kLdsBytes, "LDS budget");
+static_assert(kLdsBytes <= 160 * 1024 && kWaves * 32 * (kWaveCols * 4 + kEpiloguePadBytes) <= kLdsBytes, "LDS budget");
 
 // ---- LDS layouts ---------------------------------------------------------------------------------------
 // K-contiguous operand, [256 rows][kBK k]: 16-byte chunk c (8 k values) of row r sits at
@@ -356,48 +356,65 @@ __device__ __forceinline__ void tile_of_block(const GemmArgs &args, int &tile_m,
 }
 
 // ---- the kernel ----------------------------------------------------------------------------------------
-// Write the wavefront's 128 x 64 accumulators through its own LDS region, 32 rows at a time: registers -> LDS as
-// [32][kEpilogueStride] floats, then every lane takes 4 consecutive columns, so one store instruction covers 4 rows
-// x 64 columns (full 128-byte lines for 2-byte outputs). Row stride 72 floats keeps both the scalar writes (two
-// row groups 4 rows apart per instruction) and the 16-byte reads free of bank conflicts.
-template <typename OutT>
-__device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds, OutT *out, int64_t stride,
-                                           int rows_valid, int cols_valid, bool accumulate, int wave, int lane) {
-    constexpr int kLanesPerRow = kWaveCols / 4, kRowsPerStore = 64 / kLanesPerRow;
+// Write the wavefront's 128 x 128 accumulators through its own LDS region, 32 rows at a time. The MFMAs are issued
+// with the operands swapped (rhs fragment first), so a lane holds, of each 32 x 32 accumulator, one row and four
+// groups of four consecutive columns. Values are rounded to the output type first (unless they are to be added to
+// what `out` holds: then they stay fp32 and are rounded once after the addition), a group goes to LDS as one 8- or
+// 16-byte write, and the staged rows are read back as 16-byte chunks in row-major order, all reads of a 32-row block
+// before the first store, so that a store instruction covers full 256-byte row segments.
+template <typename OutT, bool kAccumulate>
+__device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds, OutT *out,
+                                           int64_t stride, int rows_valid, int cols_valid, int wave, int lane) {
+    using StageT = std::conditional_t<kAccumulate, float, OutT>;
+    constexpr int kChunk = 16 / sizeof(StageT);         // elements per 16-byte chunk
+    constexpr int kLanesPerRow = kWaveCols / kChunk;    // 16 or 32
+    constexpr int kRowsPerRead = 64 / kLanesPerRow;     // 4 or 2
+    constexpr int kReads = 32 / kRowsPerRead;           // 8 or 16
+    constexpr int kRowBytes = kWaveCols * sizeof(StageT) + kEpiloguePadBytes;
     const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
-    FM_LDS(float) *staging = reinterpret_cast<FM_LDS(float) *>(lds) + wave * (32 * kEpilogueStride);
-    const int column = (lane % kLanesPerRow) * 4;  // within the wavefront's columns
-    const int column_in_tile = wave_n * kWaveCols + column;
-    // cols_valid is a multiple of 8, so a group of 4 columns is valid or not as a whole.
+    FM_LDS(char) *staging = lds + wave * (32 * kRowBytes);
+    FM_LDS(char) *write_base = staging + (lane & 31) * kRowBytes + (lane >> 5) * 4 * sizeof(StageT);
+    const int read_row = lane / kLanesPerRow, read_column = (lane % kLanesPerRow) * kChunk;
+    FM_LDS(char) *read_base = staging + read_row * kRowBytes + read_column * sizeof(StageT);
+    const int column_in_tile = wave_n * kWaveCols + read_column;
+    // cols_valid is a multiple of 8, so a chunk of 4 or 8 columns is valid or not as a whole.
     const bool column_ok = column_in_tile < cols_valid;
+    const int first_row = wave_m * kWaveRows + read_row;
+    OutT *pointer = out + first_row * stride + column_in_tile;
 #pragma unroll
     for (int i = 0; i < kTilesM; ++i) {
 #pragma unroll
         for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v)
-                staging[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * kEpilogueStride + j * 32 + (lane & 31)] =
-                    acc[i][j][v];
+            for (int g = 0; g < 4; ++g) {
+                Vec16x4<StageT> group;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) group.v[c] = from_float<StageT>(acc[i][j][4 * g + c]);
+                using Raw = std::conditional_t<sizeof(StageT) == 4, u32x4_t, u32x2_t>;
+                *reinterpret_cast<FM_LDS(Raw) *>(write_base + (j * 32 + 8 * g) * sizeof(StageT)) =
+                    __builtin_bit_cast(Raw, group);
+            }
         // Only this wavefront touches its staging region and the LDS executes a wavefront's operations in order,
         // so no barrier is needed; the empty asm only keeps the compiler from moving accesses across the phases.
         asm volatile("" ::: "memory");
+        u32x4_t staged[kReads];
 #pragma unroll
-        for (int t = 0; t < 32 / kRowsPerStore; ++t) {
-            const int staged_row = t * kRowsPerStore + lane / kLanesPerRow;
-            const int row = wave_m * kWaveRows + i * 32 + staged_row;
-            const f32x4_t value = *reinterpret_cast<FM_LDS(f32x4_t) *>(staging + staged_row * kEpilogueStride + column);
-            if (row < rows_valid && column_ok) {
-                Vec16x4<OutT> packed;
-                OutT *pointer = out + row * stride + column_in_tile;
-                if (accumulate) {
-                    packed = *reinterpret_cast<const Vec16x4<OutT> *>(pointer);
+        for (int t = 0; t < kReads; ++t)
+            staged[t] = *reinterpret_cast<FM_LDS(u32x4_t) *>(read_base + t * kRowsPerRead * kRowBytes);
+#pragma unroll
+        for (int t = 0; t < kReads; ++t) {
+            const int row_in_wave = i * 32 + t * kRowsPerRead;
+            if (first_row + row_in_wave < rows_valid && column_ok) {
+                OutT *target = pointer + row_in_wave * stride;
+                if constexpr (kAccumulate) {
+                    const f32x4_t value = __builtin_bit_cast(f32x4_t, staged[t]);
+                    Vec16x4<OutT> packed = *reinterpret_cast<const Vec16x4<OutT> *>(target);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) packed.v[c] = from_float<OutT>(value[c] + to_float(packed.v[c]));
+                    store_streaming(target, packed);
                 } else {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) packed.v[c] = from_float<OutT>(value[c]);
+                    __builtin_nontemporal_store(staged[t], reinterpret_cast<u32x4_t *>(target));
                 }
-                store_streaming(pointer, packed);
             }
         }
         asm volatile("" ::: "memory");
@@ -523,7 +540,7 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
 #pragma unroll
             for (int m = 0; m < kTilesM * kTilesN; ++m) {
                 const int i = m / kTilesN, j = m % kTilesN;
-                acc[i][j] = Mfma<T>::run(frag_a[i], frag_b[kstep & 1][j], acc[i][j]);
+                acc[i][j] = Mfma<T>::run(frag_b[kstep & 1][j], frag_a[i], acc[i][j]);  // transposed, see store_tile
                 if (m < kTilesN) {
                     read_rhs_fragment(next_slot, next_kstep, (kstep + 1) & 1, m);
                 } else if (j == 0 || m == kTilesM * kTilesN - 1) {
@@ -586,15 +603,17 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     const bool accumulate = args.accumulate != 0;
     if (accumulate && num_slices == 0) return;  // nothing to add
     __syncthreads();  // all wavefronts are done reading operand slices; LDS becomes the staging area
-    if (args.out_dtype == FM_DTYPE_F32)
-        store_tile(acc, lds, static_cast<float *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
-                   work.cols_valid, accumulate, wave, lane);
-    else if (args.out_dtype == FM_DTYPE_BF16)
-        store_tile(acc, lds, static_cast<bf16_t *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
-                   work.cols_valid, accumulate, wave, lane);
-    else
-        store_tile(acc, lds, static_cast<f16_t *>(args.out) + work.out_offset, args.out_stride_row, work.rows_valid,
-                   work.cols_valid, accumulate, wave, lane);
+    auto store = [&](auto *out) {
+        if (accumulate)
+            store_tile<std::remove_pointer_t<decltype(out)>, true>(acc, lds, out + work.out_offset, args.out_stride_row,
+                                                                   work.rows_valid, work.cols_valid, wave, lane);
+        else
+            store_tile<std::remove_pointer_t<decltype(out)>, false>(acc, lds, out + work.out_offset, args.out_stride_row,
+                                                                    work.rows_valid, work.cols_valid, wave, lane);
+    };
+    if (args.out_dtype == FM_DTYPE_F32) store(static_cast<float *>(args.out));
+    else if (args.out_dtype == FM_DTYPE_BF16) store(static_cast<bf16_t *>(args.out));
+    else store(static_cast<f16_t *>(args.out));
 }
 
 // ---- host side -----------------------------------------------------------------------------------------
