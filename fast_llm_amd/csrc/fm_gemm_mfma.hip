@@ -1,11 +1,11 @@
 // Grouped matrix products on the gfx950 matrix cores (bf16 / fp16 operands, fp32 accumulation).
 //
 // One workgroup = 4 wavefronts = one 256 x 256 tile of `out`, reduced one K-slice (kBK = 64 elements) at a time:
-//   * A round trip to L2/HBM (~1.5 us under load) takes about two K-slices of multiplying, and LDS only has room
-//     for two 64 KiB slices, so the slices in flight live in registers: every lane keeps two sets of 16 x 16-byte
-//     global loads outstanding (slices t+2 and t+3, 128 KiB per workgroup) while slice t is multiplied from LDS
-//     and slice t+1 is written from registers into the other LDS slot. One barrier per slice, placed before the last
-//     K-step of a slice, whose MFMAs overlap the first fragment reads of the next slice.
+//   * A round trip to L2/HBM under load takes about two K-slices of multiplying, and LDS only has room for two
+//     64 KiB slices, so the slices in flight live in registers: every lane keeps two sets of 16 x 16-byte global loads
+//     outstanding (slices t+2 and t+3, 128 KiB per workgroup) while slice t is multiplied from LDS and slice t+1 is
+//     written from registers into the other LDS slot. One barrier per slice, placed before the last K-step of a
+//     slice, whose MFMAs overlap the first fragment reads of the next slice.
 //   * An operand may be contiguous along K (activations [rows, K], `weight.t()`) or along its other axis
 //     (`weight` [K, N], `activations.t()`). K-contiguous tiles are stored [row][K] and read as 128-bit MFMA
 //     fragments; the others are stored [K][row] as they lie in memory and read with the LDS transpose load
@@ -14,16 +14,18 @@
 //   * Wavefronts form a 2 x 2 grid, one per SIMD, each owns 128 x 128 of the tile as 4 x 4 accumulators of
 //     v_mfma_f32_32x32x16 (256 accumulation registers per lane; the other 256 hold the in-flight slices and the
 //     fragments). A single wavefront keeps the matrix pipe busy as long as its MFMAs are back to back, so every
-//     K-step is scheduled as "one MFMA, one memory instruction in its shadow" (sched_group_barrier).
+//     K-step is a fixed sequence of "one MFMA, one memory instruction in its shadow".
 //   * Tiles never straddle experts: the row tiles of an expert are enumerated from `expert_ends` on the device
-//     (ceil(rows_e / 256) each), a last partial tile loads clamped rows and stores only its valid rows, so any
-//     padding multiple works and phantom rows past the last expert are never touched. For the row-sparse product
-//     the reduction runs over [begin_e, pad_begin_e); what a K-slice holds outside that range is zeroed in LDS
-//     before it is multiplied (zero-fill, not multiply-by-zero, so NaN in padding rows cannot leak).
-//   * The tile is written through LDS: accumulators are laid out row-major per wavefront and stored as 16-byte
-//     vectors, one full 128-byte line of bf16 per row and wavefront.
-//   * Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are renumbered so every XCD works
-//     on a contiguous run of tiles (8 row tiles per column tile) and re-reads operands from its own L2.
+//     (ceil(rows_e / 256) each), a last partial tile stores only its valid rows, so any padding multiple works and
+//     phantom rows past the last expert are never touched. For the row-sparse product the reduction runs over
+//     [begin_e, pad_begin_e); what a K-slice holds outside that range is zeroed in LDS before it is multiplied
+//     (zero-fill, not multiply-by-zero, so NaN in padding rows cannot leak).
+//   * The loop has no branch around a transfer: the range of the buffer descriptors makes loads past the last slice
+//     (and rows past a partial tile of a K-contiguous operand) return zeros.
+//   * The tile is written through LDS, already rounded to the output type, as 16-byte streaming stores that cover
+//     full 256-byte row segments.
+//   * Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are renumbered so that the tiles an XCD
+//     runs at the same time are 8 row tiles x 4 column tiles that re-read operands from its own L2.
 // Results are deterministic: one workgroup per output tile, fixed summation order, no atomics.
 #include <type_traits>
 
@@ -337,15 +339,19 @@ __device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int tile_m, i
     return true;
 }
 
-// Hardware workgroup id -> (row tile, column tile): contiguous runs per XCD, 8 row tiles per column tile.
-__device__ __forceinline__ void tile_of_block(const GemmArgs &args, int &tile_m, int &tile_n) {
-    constexpr int kXcds = 8, kGroupRows = 8;
+// Hardware workgroup id -> (row tile, column tile). The hardware hands consecutive workgroup ids to the 8 XCDs in
+// turn, so the 32 CUs of XCD x run the ids x, x + 8, x + 16, ... in that order. Those are mapped to chunks of 32
+// consecutive logical tiles, chunk c going to XCD c % 8: the tiles an XCD runs at the same time are then one chunk,
+// i.e. 8 row tiles x 4 column tiles that share operand panels in that XCD's L2, while consecutive chunks go to
+// different XCDs, so that experts with many and with few tokens (long and short tiles of the row-sparse product)
+// are spread over all of them. Returns false for the ids that pad the grid to whole rounds of chunks.
+constexpr int kXcds = 8, kGroupRows = 8, kChunkTiles = 32;
+__device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int &tile_m, int &tile_n) {
     const int total = args.tiles_m * args.tiles_n;
     const int pid = blockIdx.x;
-    const int per_xcd = (total + kXcds - 1) / kXcds;
-    const int tall = total % kXcds == 0 ? kXcds : total % kXcds;
     const int xcd = pid % kXcds, local = pid / kXcds;
-    const int logical = xcd < tall ? xcd * per_xcd + local : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
+    const int logical = ((local / kChunkTiles) * kXcds + xcd) * kChunkTiles + local % kChunkTiles;
+    if (logical >= total) return false;
     const int width = kGroupRows * args.tiles_n;
     const int group = logical / width;
     const int first_m = group * kGroupRows;
@@ -353,6 +359,7 @@ __device__ __forceinline__ void tile_of_block(const GemmArgs &args, int &tile_m,
     const int in_group = logical - group * width;
     tile_m = first_m + in_group % group_rows;
     tile_n = in_group / group_rows;
+    return true;
 }
 
 // ---- the kernel ----------------------------------------------------------------------------------------
@@ -428,9 +435,8 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);  // C-style: address-space cast
 
     int tile_m, tile_n;
-    tile_of_block(args, tile_m, tile_n);
     TileWork work;
-    if (!resolve_tile(args, tile_m, tile_n, work)) return;
+    if (!tile_of_block(args, tile_m, tile_n) || !resolve_tile(args, tile_m, tile_n, work)) return;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -627,7 +633,10 @@ static int launch_instance(const GemmArgs &args, hipStream_t stream) {
         if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
         configured = true;
     }
-    kernel<<<args.tiles_m * args.tiles_n, kMfmaThreads, kLdsBytes, stream>>>(args);
+    // Whole rounds of one chunk per XCD; the surplus workgroups find no tile and exit.
+    constexpr int kRound = kXcds * kChunkTiles;
+    const int grid = (args.tiles_m * args.tiles_n + kRound - 1) / kRound * kRound;
+    kernel<<<grid, kMfmaThreads, kLdsBytes, stream>>>(args);
     return FM_OK;
 }
 
@@ -675,7 +684,7 @@ int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream) {
         args.tiles_m = static_cast<int>((args.rows + kTile - 1) / kTile + (args.expert_ends ? args.num_experts : 0));
     }
     args.tiles_n = static_cast<int>((args.cols + kTile - 1) / kTile);
-    if (static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31))
+    if (static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31) - 256)
         return fail(FM_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
     return dtype == FM_DTYPE_BF16 ? launch_layout<bf16_t>(args, stream) : launch_layout<f16_t>(args, stream);
 }
