@@ -236,3 +236,69 @@ def test_results_are_bit_identical_from_run_to_run(device):
         )
         for a, b in zip(first, again):
             assert torch.equal(a, b)
+
+
+def _ragged_case(seed: int, experts: int, pad: int = 128):
+    """Random expert sizes, some empty, some one token, padded to `pad`; plus phantom rows after the last expert."""
+    generator = torch.Generator().manual_seed(seed)
+    tokens = torch.randint(0, 700, (experts,), generator=generator)
+    tokens[torch.randint(0, experts, (max(1, experts // 8),), generator=generator)] = 0
+    tokens[int(torch.randint(0, experts, (1,), generator=generator))] = 1
+    padded = (tokens + pad - 1) // pad * pad
+    ends = torch.cumsum(padded, 0)
+    return {
+        "expert_ends": ends.tolist(),
+        "tokens_per_expert": tokens.tolist(),
+        "phantom_rows": pad * 2,
+    }
+
+
+# (experts, reduction size, per-expert size): more experts than a wavefront has lanes, an odd number of 64-wide
+# reduction slices, partial row and column tiles, more tiles than one round of workgroups.
+@pytest.mark.parametrize(("experts", "dense_dim", "sparse_dim"), [(70, 192, 264), (9, 320, 576), (130, 64, 72)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_kernel_on_ragged_experts(experts, dense_dim, sparse_dim, dtype, device):
+    case = _ragged_case(experts + dense_dim, experts)
+    oracle_map = fixture_sparse_map(case)
+    oracle_map.num_rows = case["expert_ends"][-1] + case["phantom_rows"]
+    sparse_map = to_device_map(oracle_map, device, torch.int32)
+    used = _used_rows(oracle_map)
+    real = oracle_map.real_row_mask()
+    generator = torch.Generator().manual_seed(11)
+    tolerance = _MAX_REL[dtype]
+
+    # Row-padded storage: the kernel must follow the strides.
+    def strided(rows, columns):
+        return _normal(rows, columns + 24, dtype, generator)[:, :columns]
+
+    x, weight = strided(oracle_map.num_rows, dense_dim), strided(experts * sparse_dim, dense_dim)
+    y = strided(oracle_map.num_rows, sparse_dim)
+    x_gpu, y_gpu, weight_gpu = (
+        torch.empty(t.size(0), t.size(1) + 24, dtype=dtype, device=device)[:, : t.size(1)] for t in (x, y, weight)
+    )
+    x_gpu.copy_(x), y_gpu.copy_(y), weight_gpu.copy_(weight)
+    assert not x_gpu.is_contiguous()
+
+    out = torch.full((oracle_map.num_rows, sparse_dim), 5.0, dtype=dtype, device=device)
+    output_sparse_matmul(x_gpu, weight_gpu.t(), sparse_map, out)
+    expected = moe_oracle.output_sparse_matmul(x, weight.t(), oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+    assert (out[used:] == 5.0).all()
+
+    out = input_inner_sparse_matmul(y_gpu, weight_gpu, sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(y, weight, oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+
+    y_poisoned, x_poisoned = y_gpu.clone(), x_gpu.clone()
+    y_poisoned[~real.to(device)] = float("nan")
+    x_poisoned[~real.to(device)] = float("nan")
+    for out_dtype in (dtype, torch.float32):
+        out = torch.full((experts * sparse_dim, dense_dim), 3.0, dtype=out_dtype, device=device)
+        input_row_sparse_matmul(y_poisoned.t(), x_poisoned, sparse_map, out=out)
+        expected = moe_oracle.input_row_sparse_matmul(
+            y.t(), x, oracle_map, out=torch.zeros(out.shape, dtype=out_dtype)
+        )
+        assert torch.isfinite(out).all()
+        assert max_rel_err(out.cpu(), expected) <= tolerance
+        input_row_sparse_matmul(y_poisoned.t(), x_poisoned, sparse_map, out=out, accumulate=True)
+        assert max_rel_err(out.cpu(), 2 * expected.float()) <= tolerance
