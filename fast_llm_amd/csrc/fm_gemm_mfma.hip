@@ -1,20 +1,22 @@
 // Grouped matrix products on the gfx950 matrix cores (bf16 / fp16 operands, fp32 accumulation).
 //
 // One workgroup = 4 wavefronts = one 256 x 256 tile of `out`, reduced one K-slice (kBK = 64 elements) at a time:
-//   * A round trip to L2/HBM under load takes about two K-slices of multiplying, and LDS only has room for two
-//     64 KiB slices, so the slices in flight live in registers: every lane keeps two sets of 16 x 16-byte global loads
-//     outstanding (slices t+2 and t+3, 128 KiB per workgroup) while slice t is multiplied from LDS and slice t+1 is
-//     written from registers into the other LDS slot. One barrier per slice, placed before the last K-step of a
-//     slice, whose MFMAs overlap the first fragment reads of the next slice.
+//   * Writing LDS from registers is the scarcest resource (ds_write_b128 sustains about a third of the LDS read rate),
+//     so only the rhs slices take that route: every lane keeps two sets of 8 x 16-byte global loads outstanding (rhs
+//     slices t+2 and t+3) while slice t is multiplied from LDS and slice t+1 is written from registers into the
+//     other rhs slot. The lhs slices are loaded straight into LDS (`buffer_load ... lds`), which needs a third slot
+//     because a slot that is being filled cannot be read: 3 lhs + 2 rhs slots of 32 KiB = all 160 KiB of LDS.
+//     One barrier per slice, placed before the last K-step of a slice, whose MFMAs overlap the first fragment reads
+//     of the next slice.
 //   * An operand may be contiguous along K (activations [rows, K], `weight.t()`) or along its other axis
 //     (`weight` [K, N], `activations.t()`). K-contiguous tiles are stored [row][K] and read as 128-bit MFMA
 //     fragments; the others are stored [K][row] as they lie in memory and read with the LDS transpose load
 //     `ds_read_b64_tr_b16`, which hands every lane four consecutive K values of one row. Both layouts are
 //     XOR-swizzled so that the 128-bit writes and the fragment reads hit all 64 banks.
 //   * Wavefronts form a 2 x 2 grid, one per SIMD, each owns 128 x 128 of the tile as 4 x 4 accumulators of
-//     v_mfma_f32_32x32x16 (256 accumulation registers per lane; the other 256 hold the in-flight slices and the
-//     fragments). A single wavefront keeps the matrix pipe busy as long as its MFMAs are back to back, so every
-//     K-step is a fixed sequence of "one MFMA, one memory instruction in its shadow".
+//     v_mfma_f32_32x32x16 (256 accumulation registers per lane). A single wavefront keeps the matrix pipe busy as
+//     long as its MFMAs are back to back, so every K-step is a fixed sequence of "one MFMA, one memory instruction
+//     in its shadow".
 //   * Tiles never straddle experts: the row tiles of an expert are enumerated from `expert_ends` on the device
 //     (ceil(rows_e / 256) each), a last partial tile stores only its valid rows, so any padding multiple works and
 //     phantom rows past the last expert are never touched. For the row-sparse product the reduction runs over
@@ -78,9 +80,10 @@ constexpr int kTile = 256;
 constexpr int kWavesM = 2, kWavesN = 2;  // wavefront grid over the tile
 constexpr int kWaves = kWavesM * kWavesN, kMfmaThreads = 64 * kWaves;
 constexpr int kBK = 64;      // K elements per slice (32 or 64)
-constexpr int kStages = 2;   // LDS slots
+constexpr int kStages = 2;   // LDS slots of the rhs operand (filled through registers)
+constexpr int kLhsStages = 3;  // LDS slots of the lhs operand (filled by direct-to-LDS loads)
 constexpr int kOperandBytes = kTile * kBK * 2;  // one operand slice in LDS, same size in either layout
-constexpr int kLdsBytes = 2 * kStages * kOperandBytes;  // the lhs slots, then the rhs slots
+constexpr int kLdsBytes = (kStages + kLhsStages) * kOperandBytes;  // the rhs slots, then the lhs slots
 constexpr int kWaveRows = kTile / kWavesM, kWaveCols = kTile / kWavesN;  // a wavefront's part of the tile
 constexpr int kTilesM = kWaveRows / 32, kTilesN = kWaveCols / 32;        // in 32x32 MFMA accumulators
 constexpr int kChunksPerRow = kBK / 8;          // 16-byte chunks of a K-major row
@@ -183,6 +186,23 @@ struct TileLoader {
     __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand]) {
 #pragma unroll
         for (int j = 0; j < kLoadsPerOperand; ++j) load_one(regs, j);
+    }
+
+    // The same chunk straight into LDS (`buffer_load ... lds`): lane l's 16 bytes land at M0 + 16 l, i.e. in this
+    // lane's chunk slot of the operand slot that starts at LDS byte address `slot_address`; lanes outside the
+    // descriptor's range bring zeros. The compiler does not see this load: whoever reads the slot counts the loads
+    // issued since (`s_waitcnt vmcnt`) and passes a barrier first.
+    __device__ __forceinline__ void load_direct(int slot_address, int j) {
+        const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char *>(uniform_pointer(fetch_base)), 0,
+            static_cast<int>(__builtin_amdgcn_readfirstlane(num_records)), kBufferResourceFlags);
+        const uint32_t lane_offset = offset[j & 1] + static_cast<uint32_t>(j >> 1) * pair_stride;
+        const int block_address = __builtin_amdgcn_readfirstlane(slot_address + (lds_offset & ~1023) + j * 1024);
+        // M0 is not handed out by the register allocator and nothing else in this file uses it.
+        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :
+                     : "s"(block_address), "v"(lane_offset), "s"(resource)
+                     : "memory");
     }
 
     // Write a landed slice (or its chunk j) into LDS.
@@ -472,138 +492,150 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     // ---- the software pipeline --------------------------------------------------------------------------
-    // Slice s travels through register set s % 2 and ends in LDS slot s % 2. A slice is moved in kBK / 16 chunk
-    // groups (group g = loads g * kLoadsPerStep ..), one group per K-step. During iteration t (multiplying slice t):
-    //   K-steps 0..2 : groups 1..3 of slice t + 1 go registers -> LDS, their registers are refilled from slice t + 3;
-    //   barrier      : slice t + 1 is complete and visible; nobody reads the slot of slice t any more except through
-    //                  fragments already in registers (those of K-step 3 were read during K-step 2);
-    //   K-step 3     : group 0 of slice t + 2 goes to the slot slice t just left, refill from slice t + 4; the
-    //                  fragments of K-step 0 of slice t + 1 are read.
-    // The pipeline has no branch around a transfer, which lets the compiler guard a register set with vmcnt(N > 0)
-    // instead of draining the queue: loads past the last slice bring zeros.
-    u32x4_t lhs_regs[2][kLoadsPerOperand], rhs_regs[2][kLoadsPerOperand];
-    u32x4_t frag_a[kTilesM], frag_b[2][kTilesN];
+    // LDS writes from registers are the scarcest resource of this kernel (ds_write_b128 sustains ~78 bytes per cycle
+    // and CU, a third of the read rate), so only the rhs operand takes that route; the lhs operand is loaded
+    // straight into LDS. A slot being filled that way cannot be read, hence three lhs slots and two rhs slots
+    // (160 KiB). During iteration t (multiplying slice t; r = slot t % 2, register set t % 2; l = slot t % 3):
+    //   rhs, K-steps 0..2 : chunk groups 1..3 of slice t + 1 go registers -> LDS, their registers are refilled
+    //                       from slice t + 3;
+    //   lhs, K-steps 0..2 : chunks 2..7 of slice t + 2 are loaded into lhs slot (t + 2) % 3;
+    //   barrier           : every wavefront has waited for the lhs loads of slice t + 1 it issued (all loads but
+    //                       the 12 newest have landed), so slice t + 1 is complete and visible; nobody reads the
+    //                       slots of slice t any more except through fragments already in registers (those of
+    //                       K-step 3 were read during K-step 2);
+    //   K-step 3          : rhs group 0 of slice t + 2 goes to the slot slice t just left, refill from slice t + 4;
+    //                       lhs chunks 0, 1 of slice t + 3 are loaded into the slot slice t just left; the fragments
+    //                       of K-step 0 of slice t + 1 are read.
+    // Four loads per K-step, each with three quarters of a slice or more to land (measured: capping the loads in
+    // flight at half a slice costs nothing). There is no branch around a transfer, which lets the compiler guard a
+    // register set with vmcnt(N > 0) instead of draining the queue: loads past the last slice bring zeros. The
+    // compiler's counts do not include the direct loads, which only makes its waits stricter.
+    u32x4_t rhs_regs[2][kLoadsPerOperand];
+    u32x4_t frag_a[2][kTilesM], frag_b[2][kTilesN];
     constexpr int kSteps = kBK / 16;
-    // Slice s sits in slot s % 2 of either operand. Slots are passed around as compile-time constants so that they
-    // end up in the immediate offsets of the LDS instructions.
-    auto lhs_slot = [&](int slot) { return lds + slot * kOperandBytes; };
-    auto rhs_slot = [&](int slot) { return lds + (kStages + slot) * kOperandBytes; };
-    int lhs_frag[4], rhs_frag[4];
+    constexpr int kLhsBase = kStages * kOperandBytes;  // LDS byte address of lhs slot 0; the rhs slots start at 0
+    auto rhs_slot = [&](int slot) { return lds + slot * kOperandBytes; };
+    // LDS byte addresses of the lhs slots of slices t, t + 1, t + 2 (wave-uniform, rotated after every slice) and the
+    // fragment addresses of this lane in the first two.
+    int lhs_now = kLhsBase, lhs_next = kLhsBase + kOperandBytes, lhs_after = kLhsBase + 2 * kOperandBytes;
+    int lhs_frag0[4], lhs_frag[4], lhs_frag_next[4], rhs_frag[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        lhs_frag[q] = fragment_base<kLhsContiguousK>(wave_m * kWaveRows, q, lane);
-        rhs_frag[q] = kStages * kOperandBytes + fragment_base<kRhsContiguousK>(wave_n * kWaveCols, q, lane);
+        lhs_frag0[q] = fragment_base<kLhsContiguousK>(wave_m * kWaveRows, q, lane);
+        lhs_frag[q] = lhs_frag0[q] + lhs_now;
+        lhs_frag_next[q] = lhs_frag0[q] + lhs_next;
+        rhs_frag[q] = fragment_base<kRhsContiguousK>(wave_n * kWaveCols, q, lane);
     }
-    // The rhs fragments of a K-step are all in use until its last MFMAs, so they are double-buffered; an lhs fragment
-    // is only used by kTilesN consecutive MFMAs and is re-read for the next K-step right after them.
     auto read_rhs_fragment = [&](int slot, int kstep, int buffer, int j) {
         frag_b[buffer][j] = load_fragment<kRhsContiguousK>(lds, rhs_frag, slot, j, kstep);
     };
-    auto read_lhs_fragment = [&](int slot, int kstep, int i) {
-        frag_a[i] = load_fragment<kLhsContiguousK>(lds, lhs_frag, slot, i, kstep);
+    auto read_lhs_fragment = [&](bool next_slice, int kstep, int buffer, int i) {
+        frag_a[buffer][i] = next_slice ? load_fragment<kLhsContiguousK>(lds, lhs_frag_next, 0, i, kstep)
+                                       : load_fragment<kLhsContiguousK>(lds, lhs_frag, 0, i, kstep);
     };
-    auto read_fragments = [&](int slot, int kstep, int buffer) {
-#pragma unroll
-        for (int j = 0; j < kTilesN; ++j) read_rhs_fragment(slot, kstep, buffer, j);
-#pragma unroll
-        for (int i = 0; i < kTilesM; ++i) read_lhs_fragment(slot, kstep, i);
-    };
-    auto mask_slice = [&](int slice, int slot) {
+    auto mask_slice = [&](int slice, int lhs_address, int slot) {
         if constexpr (kMasked) {
             const int k0 = static_cast<int>(k_first) + slice * kBK;
             if (slice < num_slices && (k0 < work.k_lo || k0 + kBK > work.k_hi)) {  // wave-uniform
-                mask_tile<kLhsContiguousK>(lhs_slot(slot), k0, work.k_lo, work.k_hi);
+                mask_tile<kLhsContiguousK>(lds + lhs_address, k0, work.k_lo, work.k_hi);
                 mask_tile<kRhsContiguousK>(rhs_slot(slot), k0, work.k_lo, work.k_hi);
                 __syncthreads();
             }
         }
     };
-    // `next_set` holds slice t + 1, `other_set` slice t + 2.
-    // A K-step is 16 slots of "one MFMA, then one memory instruction in its shadow" (an MFMA keeps the matrix pipe busy
-    // for 32 cycles; a clump of LDS/global instructions longer than that leaves it idle). The order is pinned with a
-    // scheduling barrier after every slot, because what a fragment read may overtake decides how long before its use
-    // it is issued: left to itself the scheduler reads the lhs fragment of the first MFMAs of a K-step last.
-    //   slots 0..3       rhs fragments 0..3 of the next K-step (other fragment buffer)
-    //   slots 4, 8, 12   lhs fragments 0, 1, 2 of the next K-step, each right after the last MFMA of its predecessor
-    //   slots 5, 6, 9, 10        registers -> LDS (lhs, rhs of chunk 0, then of chunk 1 of the group)
-    //   slots 7, 11, 13, 14      refill of the same registers from two slices further on, in the order of their use
-    //   slot 15          lhs fragment 3 of the next K-step
-    // so every fragment is issued at least 12 MFMAs before its first use.
+    // A K-step is 16 slots of "one MFMA, then at most one memory instruction in its shadow" (an MFMA keeps the matrix
+    // pipe busy for 32 cycles; a clump of LDS/global instructions longer than that leaves it idle), in an order pinned
+    // with a scheduling barrier after every slot:
+    //   slots 0..3     rhs fragments 0..3 of the next K-step (other fragment buffer)
+    //   slots 4..7     lhs fragments 0..3 of the next K-step
+    //   slots 8, 9     rhs registers -> LDS (chunks 0, 1 of the group)
+    //   slots 10, 11   refill of the same registers from two slices further on
+    //   slots 12, 13   two direct lhs loads
     static_assert(kTilesM == 4 && kTilesN == 4 && kLoadsPerStep == 2, "the slot table below is written for this shape");
     auto iteration = [&](int t, auto next_set, auto other_set) {
-        constexpr int kSlot = decltype(other_set)::value, kNextSlot = decltype(next_set)::value;  // of slices t, t + 1
+        constexpr int kSlot = decltype(other_set)::value, kNextSlot = decltype(next_set)::value;  // rhs, of slices t, t + 1
 #pragma unroll
         for (int kstep = 0; kstep < kSteps; ++kstep) {
-            const int next_slot = kstep + 1 < kSteps ? kSlot : kNextSlot, next_kstep = (kstep + 1) % kSteps;
-            // The chunk group that moves during this K-step: groups 1..3 of slice t + 1 (refilled from slice t + 3),
-            // then group 0 of slice t + 2 (refilled from slice t + 4).
+            const bool last = kstep + 1 == kSteps;
+            const int next_slot = last ? kNextSlot : kSlot, next_kstep = (kstep + 1) % kSteps;
+            const int buffer = kstep & 1;
+            // The rhs chunk group that moves during this K-step: groups 1..3 of slice t + 1 (refilled from slice
+            // t + 3), then group 0 of slice t + 2 (refilled from slice t + 4).
             const int group = (kstep + 1) % kSteps;
-            const int set = kstep + 1 < kSteps ? kNextSlot : kSlot, moved_slot = set;
-            if (kstep == kSteps - 1) {
+            const int set = last ? kSlot : kNextSlot, moved_slot = set;
+            // The lhs chunks loaded during this K-step: 2..7 of slice t + 2, then 0, 1 of slice t + 3.
+            const int lhs_chunk = 2 * group, lhs_target = last ? lhs_now : lhs_after;
+            if (last) {
                 load_lhs.advance();
                 load_rhs.advance();
             }
 #pragma unroll
             for (int m = 0; m < kTilesM * kTilesN; ++m) {
                 const int i = m / kTilesN, j = m % kTilesN;
-                acc[i][j] = Mfma<T>::run(frag_b[kstep & 1][j], frag_a[i], acc[i][j]);  // transposed, see store_tile
-                if (m < kTilesN) {
-                    read_rhs_fragment(next_slot, next_kstep, (kstep + 1) & 1, m);
-                } else if (j == 0 || m == kTilesM * kTilesN - 1) {
-                    read_lhs_fragment(next_slot, next_kstep, j == 0 ? i - 1 : i);
-                } else if (m == 5 || m == 9) {
-                    load_lhs.store_one(lhs_regs[set], lhs_slot(moved_slot), group * kLoadsPerStep + m / 8);
-                } else if (m == 6 || m == 10) {
-                    load_rhs.store_one(rhs_regs[set], rhs_slot(moved_slot), group * kLoadsPerStep + m / 8);
-                } else if (m == 7 || m == 13) {
-                    load_lhs.load_one(lhs_regs[set], group * kLoadsPerStep + m / 8);
-                } else {  // 11, 14
-                    load_rhs.load_one(rhs_regs[set], group * kLoadsPerStep + m / 12);
-                }
+                acc[i][j] = Mfma<T>::run(frag_b[buffer][j], frag_a[buffer][i], acc[i][j]);  // transposed, see store_tile
+                if (m < 4) read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
+                else if (m < 8) read_lhs_fragment(last, next_kstep, buffer ^ 1, m - 4);
+                else if (m < 10) load_rhs.store_one(rhs_regs[set], rhs_slot(moved_slot), group * kLoadsPerStep + m - 8);
+                else if (m < 12) load_rhs.load_one(rhs_regs[set], group * kLoadsPerStep + m - 10);
+                else if (m < 14) load_lhs.load_direct(lhs_target, lhs_chunk + m - 12);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (kstep == kSteps - 2) {
+                asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // all but the loads of this iteration
                 __syncthreads();
-                mask_slice(t + 1, kNextSlot);
+                mask_slice(t + 1, lhs_next, kNextSlot);
             }
+        }
+        // On to the next slice: rotate the lhs slots.
+        const int recycled = lhs_now;
+        lhs_now = lhs_next;
+        lhs_next = lhs_after;
+        lhs_after = recycled;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            lhs_frag[q] = lhs_frag_next[q];
+            lhs_frag_next[q] = lhs_frag0[q] + lhs_next;
         }
     };
     if (num_slices > 0) {
-        // Prologue: slice 0 completely into LDS, group 0 of slice 1 as well, slices 1..3 (partly) in flight.
-        load_lhs.load(lhs_regs[0]);
+        // Prologue: slices 0 and 1 of both operands and the first pieces of the next ones on their way; slice 0
+        // landed (rhs: written to LDS), rhs group 0 of slice 1 written as well.
+#pragma unroll
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load_direct(lhs_now, j);
         load_rhs.load(rhs_regs[0]);
         load_lhs.advance();
         load_rhs.advance();
-        load_lhs.load(lhs_regs[1]);
+#pragma unroll
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load_direct(lhs_next, j);
         load_rhs.load(rhs_regs[1]);
         load_lhs.advance();
         load_rhs.advance();
-        load_lhs.store(lhs_regs[0], lhs_slot(0));
         load_rhs.store(rhs_regs[0], rhs_slot(0));
-        load_lhs.load(lhs_regs[0]);
         load_rhs.load(rhs_regs[0]);
-        load_lhs.advance();
         load_rhs.advance();
 #pragma unroll
-        for (int q = 0; q < kLoadsPerStep; ++q) {
-            load_lhs.store_one(lhs_regs[1], lhs_slot(1), q);
-            load_rhs.store_one(rhs_regs[1], rhs_slot(1), q);
-        }
+        for (int q = 0; q < kLoadsPerStep; ++q) load_rhs.store_one(rhs_regs[1], rhs_slot(1), q);
 #pragma unroll
-        for (int q = 0; q < kLoadsPerStep; ++q) {
-            load_lhs.load_one(lhs_regs[1], q);
-            load_rhs.load_one(rhs_regs[1], q);
-        }
+        for (int q = 0; q < kLoadsPerStep; ++q) load_rhs.load_one(rhs_regs[1], q);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) load_lhs.load_direct(lhs_after, q);
+        // 44 loads so far, the first 8 of them lhs slice 0: it has landed once at most 28 are outstanding.
+        asm volatile("s_waitcnt vmcnt(28)" ::: "memory");
         __syncthreads();
-        mask_slice(0, 0);
-        read_fragments(0, 0, 0);
+        mask_slice(0, lhs_now, 0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            read_rhs_fragment(0, 0, 0, q);
+            read_lhs_fragment(false, 0, 0, q);
+        }
         constexpr std::integral_constant<int, 0> set0{};
         constexpr std::integral_constant<int, 1> set1{};
-        // Two slices per trip (the register sets and LDS slots alternate); an odd count multiplies one slice of zeros.
+        // Two slices per trip (the register sets and rhs slots alternate); an odd count multiplies one slice of zeros.
         for (int t = 0; t < num_slices; t += 2) {
             iteration(t, set1, set0);
             iteration(t + 1, set0, set1);
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the zero-filling direct loads past the end still write LDS
     }
 
     const bool accumulate = args.accumulate != 0;
