@@ -1,18 +1,17 @@
 // Grouped matrix products on the gfx950 matrix cores (bf16 / fp16 operands, fp32 accumulation).
 //
 // One workgroup = 4 wavefronts = one 256 x 256 tile of `out`, reduced one K-slice (kBK = 64 elements) at a time:
-//   * Writing LDS from registers is the scarcest resource (ds_write_b128 sustains about a third of the LDS read rate),
-//     so only the rhs slices take that route: every lane keeps two sets of 8 x 16-byte global loads outstanding (rhs
-//     slices t+2 and t+3) while slice t is multiplied from LDS and slice t+1 is written from registers into the
-//     other rhs slot. The lhs slices are loaded straight into LDS (`buffer_load ... lds`), which needs a third slot
-//     because a slot that is being filled cannot be read: 3 lhs + 2 rhs slots of 32 KiB = all 160 KiB of LDS.
-//     One barrier per slice, placed before the last K-step of a slice, whose MFMAs overlap the first fragment reads
-//     of the next slice.
+//   * Operand slices are loaded straight into LDS (`buffer_load ... lds`), never through registers. A slot that is
+//     being filled cannot be read, so LDS (160 KiB = five slices of 32 KiB) is split into three lhs and two rhs
+//     slots: lhs loads run two slices ahead and are issued evenly, rhs loads are issued in the half slice after
+//     their slot is released. One barrier per slice, placed before the last K-step of a slice, whose MFMAs overlap
+//     the first fragment reads of the next slice.
 //   * An operand may be contiguous along K (activations [rows, K], `weight.t()`) or along its other axis
 //     (`weight` [K, N], `activations.t()`). K-contiguous tiles are stored [row][K] and read as 128-bit MFMA
 //     fragments; the others are stored [K][row] as they lie in memory and read with the LDS transpose load
 //     `ds_read_b64_tr_b16`, which hands every lane four consecutive K values of one row. Both layouts are
-//     XOR-swizzled so that the 128-bit writes and the fragment reads hit all 64 banks.
+//     XOR-swizzled so that the fragment reads hit all 64 banks; the swizzle is applied when choosing which 16-byte
+//     chunk a lane fetches.
 //   * Wavefronts form a 2 x 2 grid, one per SIMD, each owns 128 x 128 of the tile as 4 x 4 accumulators of
 //     v_mfma_f32_32x32x16 (256 accumulation registers per lane). A single wavefront keeps the matrix pipe busy as
 //     long as its MFMAs are back to back, so every K-step is a fixed sequence of "one MFMA, one memory instruction
@@ -23,7 +22,7 @@
 //     [begin_e, pad_begin_e); what a K-slice holds outside that range is zeroed in LDS before it is multiplied
 //     (zero-fill, not multiply-by-zero, so NaN in padding rows cannot leak).
 //   * The loop has no branch around a transfer: the range of the buffer descriptors makes loads past the last slice
-//     (and rows past a partial tile of a K-contiguous operand) return zeros.
+//     (and rows past a partial tile of a K-contiguous operand) bring zeros.
 //   * The tile is written through LDS, already rounded to the output type, as 16-byte streaming stores that cover
 //     full 256-byte row segments.
 //   * Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are renumbered so that the tiles an XCD
@@ -80,19 +79,18 @@ constexpr int kTile = 256;
 constexpr int kWavesM = 2, kWavesN = 2;  // wavefront grid over the tile
 constexpr int kWaves = kWavesM * kWavesN, kMfmaThreads = 64 * kWaves;
 constexpr int kBK = 64;      // K elements per slice (32 or 64)
-constexpr int kStages = 2;   // LDS slots of the rhs operand (filled through registers)
-constexpr int kLhsStages = 3;  // LDS slots of the lhs operand (filled by direct-to-LDS loads)
+constexpr int kStages = 2;     // LDS slots of the rhs operand
+constexpr int kLhsStages = 3;  // LDS slots of the lhs operand
 constexpr int kOperandBytes = kTile * kBK * 2;  // one operand slice in LDS, same size in either layout
 constexpr int kLdsBytes = (kStages + kLhsStages) * kOperandBytes;  // the rhs slots, then the lhs slots
 constexpr int kWaveRows = kTile / kWavesM, kWaveCols = kTile / kWavesN;  // a wavefront's part of the tile
 constexpr int kTilesM = kWaveRows / 32, kTilesN = kWaveCols / 32;        // in 32x32 MFMA accumulators
 constexpr int kChunksPerRow = kBK / 8;          // 16-byte chunks of a K-major row
 constexpr int kLoadsPerOperand = kOperandBytes / 16 / kMfmaThreads;  // 16-byte loads per lane, operand and slice
-constexpr int kLoadsPerStep = kLoadsPerOperand / (kBK / 16);        // of them moved during one K-step
 constexpr int kBufferResourceFlags = 0x00020000;  // raw buffer, 32-bit data format, no swizzle
 constexpr int kEpiloguePadBytes = 16;  // after each staged row of the epilogue; keeps 16-byte alignment and spreads
                                        // the rows over the banks
-static_assert(kBK == 64 && kLoadsPerStep >= 1 && kLoadsPerStep * (kBK / 16) == kLoadsPerOperand, "pipeline shape");
+static_assert(kBK == 64 && kLoadsPerOperand == 8, "pipeline shape");
 static_assert(kLdsBytes <= 160 * 1024 && kWaves * 32 * (kWaveCols * 4 + kEpiloguePadBytes) <= kLdsBytes, "LDS budget");
 
 // ---- LDS layouts ---------------------------------------------------------------------------------------
@@ -120,28 +118,34 @@ __device__ __forceinline__ const char *uniform_pointer(const char *pointer) {
     return reinterpret_cast<const char *>((static_cast<uint64_t>(high) << 32) | low);
 }
 
-// Loader of one operand slice: global memory -> registers -> LDS. The slice is 256 * kBK / 8 chunks of 16 bytes;
-// chunk slot p of the LDS slice is handled by lane p % 64 of wavefront (p / 64) / kLoadsPerOperand as its load
-// number (p / 64) % kLoadsPerOperand, so a wavefront writes 1 KiB of consecutive LDS per instruction.
+// Loader of one operand slice: global memory -> LDS, without passing through registers (`buffer_load ... lds`: lane
+// l of the wavefront fetches 16 bytes at its own offset and the hardware puts them at M0 + 16 l in LDS; lanes outside
+// the descriptor's range bring zeros). Writing LDS from registers instead (ds_write_b128) sustains only ~78 bytes per
+// cycle and CU, a third of the LDS read rate, and was the busiest pipe of this kernel.
+// The slice is 256 * kBK / 8 chunks of 16 bytes; chunk slot p of the LDS slice is fetched by lane p % 64 of wavefront
+// (p / 64) / kLoadsPerOperand as its load number (p / 64) % kLoadsPerOperand, so a load instruction fills 1 KiB of
+// consecutive LDS and the swizzle is applied on the global side (which chunk a lane fetches).
+// The compiler does not see these loads: whoever reads a slot counts the loads issued since (`s_waitcnt vmcnt`, loads
+// complete in order) and passes a barrier first.
 template <bool kContiguousK>
 struct TileLoader {
     const char *fetch_base;  // wave-uniform: first row of the tile, first k of the slice being fetched
     uint32_t offset[2];      // per lane, bytes from `fetch_base`, of loads 0 and 1 (fits 32 bits: checked on the host)
     uint32_t pair_stride;    // wave-uniform: bytes from load j to load j + 2 (the swizzles repeat with period 2)
-    uint32_t num_records;    // wave-uniform: lane offsets >= this read as zero
+    uint32_t num_records;    // wave-uniform: lane offsets >= this bring zeros
     int64_t step;            // bytes from one slice to the next
     int slices_left;         // slices after the one being fetched
-    int lds_offset;          // of this lane's first slot
+    int lds_offset;          // wave-uniform: of this wavefront's first 1 KiB block within an operand slot
 
     // `stride`: bytes between rows (K-contiguous) or between K-rows (row-contiguous). Rows >= valid_rows are never
-    // stored; a K-contiguous operand reads them as zero (they lie past the range of the buffer descriptor), a
-    // row-contiguous one reads in-range rows in their place.
+    // stored; a K-contiguous operand gets zeros for them (they lie past the range of the buffer descriptor), a
+    // row-contiguous one gets in-range rows in their place.
     __device__ __forceinline__ void setup(const char *tile_base, int64_t stride, int valid_rows, int num_slices,
                                           int wave, int lane) {
         static_assert(kLoadsPerOperand % 2 == 0, "loads come in (even, odd) pairs");
         fetch_base = tile_base;
         slices_left = num_slices - 1;
-        lds_offset = (wave * kLoadsPerOperand * 64 + lane) * 16;
+        lds_offset = wave * kLoadsPerOperand * 1024;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int slot = (wave * kLoadsPerOperand + j) * 64 + lane;
@@ -164,7 +168,7 @@ struct TileLoader {
     }
 
     // Move on to the next slice. Past the last slice the descriptor's range becomes empty, so that every further
-    // load brings zeros without touching memory: the pipeline can run a slice too far without a branch.
+    // load fills LDS with zeros without touching memory: the pipeline can run a slice too far without a branch.
     __device__ __forceinline__ void advance() {
         // Said to be wave-uniform once more: loop-carried values otherwise end up in vector registers.
         fetch_base = uniform_pointer(fetch_base + step);
@@ -172,49 +176,28 @@ struct TileLoader {
         num_records = __builtin_amdgcn_readfirstlane(slices_left < 0 ? 0u : num_records);
     }
 
-    // Buffer loads: scalar base (in the resource descriptor) + 32-bit lane offset, so the addresses cost two
-    // registers per operand and advancing to the next slice is scalar arithmetic.
-    // Chunk j of the slice being fetched into regs[j].
-    __device__ __forceinline__ void load_one(u32x4_t (&regs)[kLoadsPerOperand], int j) {
+    // Chunk j of the slice being fetched -> the operand slot that starts at LDS byte address `slot_address`.
+    // Buffer load: scalar base (in the resource descriptor) + 32-bit lane offset, so the addresses cost two registers
+    // per operand and advancing to the next slice is scalar arithmetic.
+    __device__ __forceinline__ void load(int slot_address, int j) {
         const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<char *>(uniform_pointer(fetch_base)), 0,
             static_cast<int>(__builtin_amdgcn_readfirstlane(num_records)), kBufferResourceFlags);
         const uint32_t lane_offset = offset[j & 1] + static_cast<uint32_t>(j >> 1) * pair_stride;
-        regs[j] = __builtin_bit_cast(
-            u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, static_cast<int>(lane_offset), 0, 0));
-    }
-    __device__ __forceinline__ void load(u32x4_t (&regs)[kLoadsPerOperand]) {
-#pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) load_one(regs, j);
-    }
-
-    // The same chunk straight into LDS (`buffer_load ... lds`): lane l's 16 bytes land at M0 + 16 l, i.e. in this
-    // lane's chunk slot of the operand slot that starts at LDS byte address `slot_address`; lanes outside the
-    // descriptor's range bring zeros. The compiler does not see this load: whoever reads the slot counts the loads
-    // issued since (`s_waitcnt vmcnt`) and passes a barrier first.
-    __device__ __forceinline__ void load_direct(int slot_address, int j) {
-        const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<char *>(uniform_pointer(fetch_base)), 0,
-            static_cast<int>(__builtin_amdgcn_readfirstlane(num_records)), kBufferResourceFlags);
-        const uint32_t lane_offset = offset[j & 1] + static_cast<uint32_t>(j >> 1) * pair_stride;
-        const int block_address = __builtin_amdgcn_readfirstlane(slot_address + (lds_offset & ~1023) + j * 1024);
+        const int block_address = __builtin_amdgcn_readfirstlane(slot_address + lds_offset + j * 1024);
         // M0 is not handed out by the register allocator and nothing else in this file uses it.
         asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      :
                      : "s"(block_address), "v"(lane_offset), "s"(resource)
                      : "memory");
     }
-
-    // Write a landed slice (or its chunk j) into LDS.
-    __device__ __forceinline__ void store_one(const u32x4_t (&regs)[kLoadsPerOperand], FM_LDS(char) * operand_lds,
-                                              int j) {
-        *reinterpret_cast<FM_LDS(u32x4_t) *>(operand_lds + lds_offset + j * 1024) = regs[j];
-    }
-    __device__ __forceinline__ void store(const u32x4_t (&regs)[kLoadsPerOperand], FM_LDS(char) * operand_lds) {
-#pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) store_one(regs, operand_lds, j);
-    }
 };
+
+// Returns once at most `kNewest` of the loads this wavefront has issued are still on their way.
+template <int kNewest>
+__device__ __forceinline__ void wait_for_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kNewest) : "memory");
+}
 
 // MFMA operand fragments (8 consecutive k of one row per lane; lane l: row l % 32, k half l / 32). A wavefront reads
 // 4 fragments (32 rows each, `i`) for each of the 4 K-steps of a slice, from either LDS slot. Thanks to the period of
@@ -492,29 +475,22 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     // ---- the software pipeline --------------------------------------------------------------------------
-    // LDS writes from registers are the scarcest resource of this kernel (ds_write_b128 sustains ~78 bytes per cycle
-    // and CU, a third of the read rate), so only the rhs operand takes that route; the lhs operand is loaded
-    // straight into LDS. A slot being filled that way cannot be read, hence three lhs slots and two rhs slots
-    // (160 KiB). During iteration t (multiplying slice t; r = slot t % 2, register set t % 2; l = slot t % 3):
-    //   rhs, K-steps 0..2 : chunk groups 1..3 of slice t + 1 go registers -> LDS, their registers are refilled
-    //                       from slice t + 3;
-    //   lhs, K-steps 0..2 : chunks 2..7 of slice t + 2 are loaded into lhs slot (t + 2) % 3;
-    //   barrier           : every wavefront has waited for the lhs loads of slice t + 1 it issued (all loads but
-    //                       the 12 newest have landed), so slice t + 1 is complete and visible; nobody reads the
-    //                       slots of slice t any more except through fragments already in registers (those of
-    //                       K-step 3 were read during K-step 2);
-    //   K-step 3          : rhs group 0 of slice t + 2 goes to the slot slice t just left, refill from slice t + 4;
-    //                       lhs chunks 0, 1 of slice t + 3 are loaded into the slot slice t just left; the fragments
-    //                       of K-step 0 of slice t + 1 are read.
-    // Four loads per K-step, each with three quarters of a slice or more to land (measured: capping the loads in
-    // flight at half a slice costs nothing). There is no branch around a transfer, which lets the compiler guard a
-    // register set with vmcnt(N > 0) instead of draining the queue: loads past the last slice bring zeros. The
-    // compiler's counts do not include the direct loads, which only makes its waits stricter.
-    u32x4_t rhs_regs[2][kLoadsPerOperand];
+    // A slot that is being filled cannot be read, and LDS (160 KiB) has room for five operand slices of 32 KiB: three
+    // lhs slots and two rhs slots. During iteration t (multiplying slice t; rhs slot t % 2, lhs slot t % 3):
+    //   K-step 0     : rhs chunks 4..7 of slice t + 1 are loaded (into the slot slice t - 1 left);
+    //   K-steps 0..2 : lhs chunks 2..7 of slice t + 2 are loaded, two per K-step, into lhs slot (t + 2) % 3;
+    //   barrier      : every wavefront has waited for all its loads but the 6 newest (the lhs loads of this
+    //                  iteration), so slice t + 1 is complete and visible; nobody reads the slots of slice t any more
+    //                  except through fragments already in registers (those of K-step 3 were read during K-step 2);
+    //   K-step 3     : rhs chunks 0..3 of slice t + 2 and lhs chunks 0, 1 of slice t + 3 are loaded into the slots
+    //                  slice t just left; the fragments of K-step 0 of slice t + 1 are read.
+    // So an lhs load has a slice or more to land and an rhs load half a slice or more (measured on the predecessor of
+    // this pipeline: capping the loads in flight at half a slice per wavefront costs nothing, a quarter costs 6 %).
+    // Fragments are double-buffered over K-steps, across slices as well. There is no branch around a transfer: loads
+    // past the last slice bring zeros.
     u32x4_t frag_a[2][kTilesM], frag_b[2][kTilesN];
     constexpr int kSteps = kBK / 16;
     constexpr int kLhsBase = kStages * kOperandBytes;  // LDS byte address of lhs slot 0; the rhs slots start at 0
-    auto rhs_slot = [&](int slot) { return lds + slot * kOperandBytes; };
     // LDS byte addresses of the lhs slots of slices t, t + 1, t + 2 (wave-uniform, rotated after every slice) and the
     // fragment addresses of this lane in the first two.
     int lhs_now = kLhsBase, lhs_next = kLhsBase + kOperandBytes, lhs_after = kLhsBase + 2 * kOperandBytes;
@@ -533,12 +509,12 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         frag_a[buffer][i] = next_slice ? load_fragment<kLhsContiguousK>(lds, lhs_frag_next, 0, i, kstep)
                                        : load_fragment<kLhsContiguousK>(lds, lhs_frag, 0, i, kstep);
     };
-    auto mask_slice = [&](int slice, int lhs_address, int slot) {
+    auto mask_slice = [&](int slice, int lhs_address, int rhs_slot) {
         if constexpr (kMasked) {
             const int k0 = static_cast<int>(k_first) + slice * kBK;
             if (slice < num_slices && (k0 < work.k_lo || k0 + kBK > work.k_hi)) {  // wave-uniform
                 mask_tile<kLhsContiguousK>(lds + lhs_address, k0, work.k_lo, work.k_hi);
-                mask_tile<kRhsContiguousK>(rhs_slot(slot), k0, work.k_lo, work.k_hi);
+                mask_tile<kRhsContiguousK>(lds + rhs_slot * kOperandBytes, k0, work.k_lo, work.k_hi);
                 __syncthreads();
             }
         }
@@ -548,23 +524,18 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     // with a scheduling barrier after every slot:
     //   slots 0..3     rhs fragments 0..3 of the next K-step (other fragment buffer)
     //   slots 4..7     lhs fragments 0..3 of the next K-step
-    //   slots 8, 9     rhs registers -> LDS (chunks 0, 1 of the group)
-    //   slots 10, 11   refill of the same registers from two slices further on
-    //   slots 12, 13   two direct lhs loads
-    static_assert(kTilesM == 4 && kTilesN == 4 && kLoadsPerStep == 2, "the slot table below is written for this shape");
-    auto iteration = [&](int t, auto next_set, auto other_set) {
-        constexpr int kSlot = decltype(other_set)::value, kNextSlot = decltype(next_set)::value;  // rhs, of slices t, t + 1
+    //   slots 8..11    in K-steps 0 and 3: four rhs loads
+    //   slots 12, 13   two lhs loads
+    static_assert(kTilesM == 4 && kTilesN == 4 && kLoadsPerOperand == 8, "the slot table below is written for this shape");
+    auto iteration = [&](int t, auto slot_constant) {
+        constexpr int kSlot = decltype(slot_constant)::value, kNextSlot = 1 - kSlot;  // rhs, of slices t, t + 1
 #pragma unroll
         for (int kstep = 0; kstep < kSteps; ++kstep) {
             const bool last = kstep + 1 == kSteps;
             const int next_slot = last ? kNextSlot : kSlot, next_kstep = (kstep + 1) % kSteps;
             const int buffer = kstep & 1;
-            // The rhs chunk group that moves during this K-step: groups 1..3 of slice t + 1 (refilled from slice
-            // t + 3), then group 0 of slice t + 2 (refilled from slice t + 4).
-            const int group = (kstep + 1) % kSteps;
-            const int set = last ? kSlot : kNextSlot, moved_slot = set;
             // The lhs chunks loaded during this K-step: 2..7 of slice t + 2, then 0, 1 of slice t + 3.
-            const int lhs_chunk = 2 * group, lhs_target = last ? lhs_now : lhs_after;
+            const int lhs_chunk = 2 * next_kstep, lhs_target = last ? lhs_now : lhs_after;
             if (last) {
                 load_lhs.advance();
                 load_rhs.advance();
@@ -573,15 +544,20 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             for (int m = 0; m < kTilesM * kTilesN; ++m) {
                 const int i = m / kTilesN, j = m % kTilesN;
                 acc[i][j] = Mfma<T>::run(frag_b[buffer][j], frag_a[buffer][i], acc[i][j]);  // transposed, see store_tile
-                if (m < 4) read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
-                else if (m < 8) read_lhs_fragment(last, next_kstep, buffer ^ 1, m - 4);
-                else if (m < 10) load_rhs.store_one(rhs_regs[set], rhs_slot(moved_slot), group * kLoadsPerStep + m - 8);
-                else if (m < 12) load_rhs.load_one(rhs_regs[set], group * kLoadsPerStep + m - 10);
-                else if (m < 14) load_lhs.load_direct(lhs_target, lhs_chunk + m - 12);
+                if (m < 4) {
+                    read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
+                } else if (m < 8) {
+                    read_lhs_fragment(last, next_kstep, buffer ^ 1, m - 4);
+                } else if (m < 12) {
+                    if (kstep == 0) load_rhs.load(kNextSlot * kOperandBytes, 4 + m - 8);
+                    else if (last) load_rhs.load(kSlot * kOperandBytes, m - 8);
+                } else if (m < 14) {
+                    load_lhs.load(lhs_target, lhs_chunk + m - 12);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (kstep == kSteps - 2) {
-                asm volatile("s_waitcnt vmcnt(12)" ::: "memory");  // all but the loads of this iteration
+                wait_for_loads<6>();
                 __syncthreads();
                 mask_slice(t + 1, lhs_next, kNextSlot);
             }
@@ -598,29 +574,21 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         }
     };
     if (num_slices > 0) {
-        // Prologue: slices 0 and 1 of both operands and the first pieces of the next ones on their way; slice 0
-        // landed (rhs: written to LDS), rhs group 0 of slice 1 written as well.
+        // Prologue: slice 0, lhs slice 1 and the first pieces of the slices after them on their way; slice 0 landed.
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load_direct(lhs_now, j);
-        load_rhs.load(rhs_regs[0]);
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load(lhs_now, j);
+#pragma unroll
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_rhs.load(0, j);
         load_lhs.advance();
         load_rhs.advance();
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load_direct(lhs_next, j);
-        load_rhs.load(rhs_regs[1]);
+        for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load(lhs_next, j);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_rhs.load(kOperandBytes, j);
         load_lhs.advance();
-        load_rhs.advance();
-        load_rhs.store(rhs_regs[0], rhs_slot(0));
-        load_rhs.load(rhs_regs[0]);
-        load_rhs.advance();
 #pragma unroll
-        for (int q = 0; q < kLoadsPerStep; ++q) load_rhs.store_one(rhs_regs[1], rhs_slot(1), q);
-#pragma unroll
-        for (int q = 0; q < kLoadsPerStep; ++q) load_rhs.load_one(rhs_regs[1], q);
-#pragma unroll
-        for (int q = 0; q < 2; ++q) load_lhs.load_direct(lhs_after, q);
-        // 44 loads so far, the first 8 of them lhs slice 0: it has landed once at most 28 are outstanding.
-        asm volatile("s_waitcnt vmcnt(28)" ::: "memory");
+        for (int j = 0; j < 2; ++j) load_lhs.load(lhs_after, j);
+        wait_for_loads<14>();  // 30 loads so far, the first 16 of them slice 0
         __syncthreads();
         mask_slice(0, lhs_now, 0);
 #pragma unroll
@@ -628,14 +596,14 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             read_rhs_fragment(0, 0, 0, q);
             read_lhs_fragment(false, 0, 0, q);
         }
-        constexpr std::integral_constant<int, 0> set0{};
-        constexpr std::integral_constant<int, 1> set1{};
-        // Two slices per trip (the register sets and rhs slots alternate); an odd count multiplies one slice of zeros.
+        constexpr std::integral_constant<int, 0> slot0{};
+        constexpr std::integral_constant<int, 1> slot1{};
+        // Two slices per trip (the rhs slots alternate); an odd count multiplies one slice of zeros.
         for (int t = 0; t < num_slices; t += 2) {
-            iteration(t, set1, set0);
-            iteration(t + 1, set0, set1);
+            iteration(t, slot0);
+            iteration(t + 1, slot1);
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the zero-filling direct loads past the end still write LDS
+        wait_for_loads<0>();  // the zero-filling loads of slices past the end still write LDS
     }
 
     const bool accumulate = args.accumulate != 0;
