@@ -411,11 +411,14 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTiles
 #pragma unroll
         for (int t = 0; t < kReads; ++t)
             staged[t] = *reinterpret_cast<FM_LDS(u32x4_t) *>(read_base + t * kRowsPerRead * kRowBytes);
+        // A running pointer, and no per-store checks when the whole tile is valid (wave-uniform).
+        auto store_rows = [&](auto whole_tile) {
+            OutT *target = pointer + static_cast<int64_t>(i) * 32 * stride;
 #pragma unroll
-        for (int t = 0; t < kReads; ++t) {
-            const int row_in_wave = i * 32 + t * kRowsPerRead;
-            if (first_row + row_in_wave < rows_valid && column_ok) {
-                OutT *target = pointer + row_in_wave * stride;
+            for (int t = 0; t < kReads; ++t, target += kRowsPerRead * stride) {
+                if constexpr (!decltype(whole_tile)::value) {
+                    if (!(first_row + i * 32 + t * kRowsPerRead < rows_valid && column_ok)) continue;
+                }
                 if constexpr (kAccumulate) {
                     const f32x4_t value = __builtin_bit_cast(f32x4_t, staged[t]);
                     Vec16x4<OutT> packed = *reinterpret_cast<const Vec16x4<OutT> *>(target);
@@ -426,7 +429,9 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTiles
                     __builtin_nontemporal_store(staged[t], reinterpret_cast<u32x4_t *>(target));
                 }
             }
-        }
+        };
+        if (rows_valid == kTile && cols_valid == kTile) store_rows(std::true_type{});
+        else store_rows(std::false_type{});
         asm volatile("" ::: "memory");
     }
 }
