@@ -32,65 +32,117 @@ __device__ __forceinline__ float load_score(const void *scores, int scores_dtype
 }
 
 // ---- dispatch ------------------------------------------------------------------------------------------
-template <typename T, bool kVector>
+// One workgroup per token. kChunks > 0: the row has at most kChunks vectors per lane, all loaded before the first
+// store (more bytes in flight per CU); kChunks = 0: any row length, one vector per lane at a time.
+template <typename T, bool kVector, int kChunks>
 __global__ __launch_bounds__(kCopyThreads) void copy_dense_to_sparse_kernel(const T *__restrict__ input,
                                                                             T *__restrict__ output, CopyArgs args) {
     constexpr int N = kVector ? Vec16<T>::N : 1;
-    const int64_t token = blockIdx.x;
+    constexpr int kPasses = kChunks > 0 ? kChunks : 1;
     const int64_t columns = args.num_columns;
-    const T *in_row = input + token * columns;
     const int k = args.experts_per_token;
-    for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns; c += static_cast<int64_t>(blockDim.x) * N) {
-        Vec16<T> value;
-        if constexpr (kVector) value = load16(in_row + c);
-        else value.v[0] = in_row[c];
+    const int64_t stride = static_cast<int64_t>(blockDim.x) * N;
+    const int64_t token = blockIdx.x;
+    for (int64_t c0 = static_cast<int64_t>(threadIdx.x) * N; c0 < columns; c0 += stride * kPasses) {
+        Vec16<T> value[kPasses];
+        const T *in_row = input + token * columns;
+#pragma unroll
+        for (int q = 0; q < kPasses; ++q) {
+            const int64_t c = c0 + q * stride;
+            if (c < columns) {
+                if constexpr (kVector) value[q] = load16(in_row + c);
+                else value[q].v[0] = in_row[c];
+            }
+        }
         for (int j = 0; j < k; ++j) {
             const int64_t row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
             if (row < 0) continue;
-            Vec16<T> scaled = value;
-            if (args.scores != nullptr) {
-                const float score = load_score(args.scores, args.scores_dtype, token * k + j);
+            const bool scaled_copy = args.scores != nullptr;
+            const float score = scaled_copy ? load_score(args.scores, args.scores_dtype, token * k + j) : 1.f;
 #pragma unroll
-                for (int i = 0; i < N; ++i) scaled.v[i] = from_float<T>(to_float(value.v[i]) * score);
+            for (int q = 0; q < kPasses; ++q) {
+                const int64_t c = c0 + q * stride;
+                if (c >= columns) continue;
+                Vec16<T> scaled = value[q];
+                if (scaled_copy) {
+#pragma unroll
+                    for (int i = 0; i < N; ++i) scaled.v[i] = from_float<T>(to_float(value[q].v[i]) * score);
+                }
+                if constexpr (kVector) store16(output + row * columns + c, scaled);
+                else output[row * columns + c] = scaled.v[0];
             }
-            if constexpr (kVector) store16(output + row * columns + c, scaled);
-            else output[row * columns + c] = scaled.v[0];
         }
+        if (kChunks > 0) break;
     }
 }
 
 // ---- combine -------------------------------------------------------------------------------------------
-template <typename T, bool kVector>
+// Slots are taken two at a time: all loads of a pair (and of all the lane's vectors) are issued before the first
+// addition; the additions keep the slot order j = 0 .. k - 1.
+template <typename T, bool kVector, int kChunks>
 __global__ __launch_bounds__(kCopyThreads) void copy_sparse_to_dense_kernel(const T *__restrict__ input,
                                                                             T *__restrict__ output, CopyArgs args) {
     constexpr int N = kVector ? Vec16<T>::N : 1;
-    const int64_t token = blockIdx.x;
+    constexpr int kPasses = kChunks > 0 ? kChunks : 1;
+    constexpr int kGroup = 2;
     const int64_t columns = args.num_columns;
     const int k = args.experts_per_token;
-    for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns; c += static_cast<int64_t>(blockDim.x) * N) {
-        float sum[N];
+    const int64_t stride = static_cast<int64_t>(blockDim.x) * N;
+    const int64_t token = blockIdx.x;
+    for (int64_t c0 = static_cast<int64_t>(threadIdx.x) * N; c0 < columns; c0 += stride * kPasses) {
+        float sum[kPasses][N];
 #pragma unroll
-        for (int i = 0; i < N; ++i) sum[i] = 0.f;
-        for (int j = 0; j < k; ++j) {
-            const int64_t row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
-            if (row < 0) continue;
-            Vec16<T> value;
-            if constexpr (kVector) value = load16(input + row * columns + c);
-            else value.v[0] = input[row * columns + c];
-            if (args.scores != nullptr) {
-                const float score = load_score(args.scores, args.scores_dtype, token * k + j);
+        for (int q = 0; q < kPasses; ++q)
 #pragma unroll
-                for (int i = 0; i < N; ++i) sum[i] += to_float(value.v[i]) * score;
-            } else {
+            for (int i = 0; i < N; ++i) sum[q][i] = 0.f;
+        for (int j0 = 0; j0 < k; j0 += kGroup) {
+            Vec16<T> value[kGroup][kPasses];
+            float score[kGroup];
+            bool present[kGroup];
 #pragma unroll
-                for (int i = 0; i < N; ++i) sum[i] += to_float(value.v[i]);
+            for (int u = 0; u < kGroup; ++u) {
+                const int j = j0 + u;
+                const int64_t row = j < k ? load_index(args.sparse_rows, args.index_dtype, token * k + j) : -1;
+                present[u] = row >= 0;
+                score[u] = 1.f;
+                if (present[u]) {
+                    if (args.scores != nullptr) score[u] = load_score(args.scores, args.scores_dtype, token * k + j);
+#pragma unroll
+                    for (int q = 0; q < kPasses; ++q) {
+                        const int64_t c = c0 + q * stride;
+                        if (c < columns) {
+                            if constexpr (kVector) value[u][q] = load16(input + row * columns + c);
+                            else value[u][q].v[0] = input[row * columns + c];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u) {
+                if (!present[u]) continue;
+#pragma unroll
+                for (int q = 0; q < kPasses; ++q) {
+                    if (args.scores != nullptr) {
+#pragma unroll
+                        for (int i = 0; i < N; ++i) sum[q][i] += to_float(value[u][q].v[i]) * score[u];
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < N; ++i) sum[q][i] += to_float(value[u][q].v[i]);
+                    }
+                }
             }
         }
-        Vec16<T> result;
 #pragma unroll
-        for (int i = 0; i < N; ++i) result.v[i] = from_float<T>(sum[i]);
-        if constexpr (kVector) store16(output + token * columns + c, result);
-        else output[token * columns + c] = result.v[0];
+        for (int q = 0; q < kPasses; ++q) {
+            const int64_t c = c0 + q * stride;
+            if (c >= columns) continue;
+            Vec16<T> result;
+#pragma unroll
+            for (int i = 0; i < N; ++i) result.v[i] = from_float<T>(sum[q][i]);
+            if constexpr (kVector) store16(output + token * columns + c, result);
+            else output[token * columns + c] = result.v[0];
+        }
+        if (kChunks > 0) break;
     }
 }
 
@@ -181,6 +233,26 @@ static int copy_threads(int64_t num_columns, int vector) {
     return static_cast<int>(threads);
 }
 
+#define FM_DEFINE_COPY_LAUNCHER(NAME, KERNEL)                                                                        \
+    template <typename T>                                                                                            \
+    static void NAME(const T *in, T *out, int64_t rows, const CopyArgs &args, bool vectorised, int chunks,          \
+                     int threads, hipStream_t stream) {                                                              \
+        if (!vectorised) KERNEL<T, false, 0><<<rows, threads, 0, stream>>>(in, out, args);                           \
+        else if (chunks <= 1) KERNEL<T, true, 1><<<rows, threads, 0, stream>>>(in, out, args);                       \
+        else if (chunks <= 2) KERNEL<T, true, 2><<<rows, threads, 0, stream>>>(in, out, args);                       \
+        else if (chunks <= 4) KERNEL<T, true, 4><<<rows, threads, 0, stream>>>(in, out, args);                       \
+        else KERNEL<T, true, 0><<<rows, threads, 0, stream>>>(in, out, args);                                        \
+    }
+FM_DEFINE_COPY_LAUNCHER(launch_dispatch, copy_dense_to_sparse_kernel)
+FM_DEFINE_COPY_LAUNCHER(launch_combine, copy_sparse_to_dense_kernel)
+#undef FM_DEFINE_COPY_LAUNCHER
+
+// Vectors of `vector` elements a lane handles when `threads` lanes share a row.
+static int chunks_per_lane(int64_t num_columns, int vector, int threads) {
+    const int64_t per_pass = static_cast<int64_t>(vector) * threads;
+    return static_cast<int>(min((num_columns + per_pass - 1) / per_pass, static_cast<int64_t>(1 << 20)));
+}
+
 static int validate_copy(const char *name, const void *a, const void *b, const void *sparse_rows, int64_t rows,
                          int64_t columns, int64_t k, int64_t rows_sparse, int dtype, int scores_dtype,
                          int index_dtype) {
@@ -211,13 +283,10 @@ extern "C" int fm_copy_dense_to_sparse(const void *input, const void *scores, co
     const int vector = 16 / dtype_size(dtype);
     const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(output);
     const int threads = copy_threads(num_columns, vectorised ? vector : 1);
+    const int chunks = chunks_per_lane(num_columns, vectorised ? vector : 1, threads);
     FM_DISPATCH_DTYPE(dtype, T, {
-        if (vectorised)
-            copy_dense_to_sparse_kernel<T, true><<<num_rows_dense, threads, 0, stream>>>(
-                static_cast<const T *>(input), static_cast<T *>(output), args);
-        else
-            copy_dense_to_sparse_kernel<T, false><<<num_rows_dense, threads, 0, stream>>>(
-                static_cast<const T *>(input), static_cast<T *>(output), args);
+        launch_dispatch<T>(static_cast<const T *>(input), static_cast<T *>(output), num_rows_dense, args, vectorised, chunks,
+                    threads, stream);
     });
     return check_launch(name);
 }
@@ -237,13 +306,10 @@ extern "C" int fm_copy_sparse_to_dense(const void *input, const void *scores, co
     const int vector = 16 / dtype_size(dtype);
     const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(output);
     const int threads = copy_threads(num_columns, vectorised ? vector : 1);
+    const int chunks = chunks_per_lane(num_columns, vectorised ? vector : 1, threads);
     FM_DISPATCH_DTYPE(dtype, T, {
-        if (vectorised)
-            copy_sparse_to_dense_kernel<T, true><<<num_rows_dense, threads, 0, stream>>>(
-                static_cast<const T *>(input), static_cast<T *>(output), args);
-        else
-            copy_sparse_to_dense_kernel<T, false><<<num_rows_dense, threads, 0, stream>>>(
-                static_cast<const T *>(input), static_cast<T *>(output), args);
+        launch_combine<T>(static_cast<const T *>(input), static_cast<T *>(output), num_rows_dense, args, vectorised, chunks,
+                    threads, stream);
     });
     return check_launch(name);
 }
