@@ -23,10 +23,7 @@ def attach_grad_buffer(weight: torch.Tensor, dtype: torch.dtype | None = None) -
     return weight
 
 
-def topk_routing(logits: torch.Tensor, experts_per_token: int) -> tuple[torch.Tensor, torch.Tensor]:
-    """Reference: mixture_of_experts.py:243-244."""
-    top_logits, top_experts = torch.topk(logits, k=experts_per_token, dim=-1)
-    return torch.softmax(top_logits, dim=-1, dtype=torch.float32), top_experts
+from fast_llm_amd.functional.routing import topk_routing  # noqa: E402  (re-exported: the layer's routing step)
 
 
 class DroplessMoEMLP(torch.nn.Module):

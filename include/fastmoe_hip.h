@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 1
+#define FM_VERSION 2
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -124,6 +124,25 @@ int fm_copy_sparse_to_dense_backward(const void *input, const void *grad_output,
                                      int64_t num_rows_dense, int64_t num_columns, int64_t num_experts_per_token,
                                      int64_t num_rows_sparse, int dtype, int scores_dtype, int out_dtype,
                                      int index_dtype, void *stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Top-k routing (the step just before the sparse map). `logits` is [num_tokens, num_experts], contiguous, of
+ * `dtype`; num_experts <= 1024, experts_per_token <= 64.
+ * --------------------------------------------------------------------------------------------------------- */
+
+/* top_experts[t, j] (int64) = expert of the j-th largest logit of token t (ties: lower expert first);
+ * scores[t, :] (fp32) = softmax over those experts_per_token logits, computed in fp32.
+ * Replaces the torch.topk + torch.softmax pair of `MixtureOfExpertMLP._topk_routing`
+ * (fast_llm/layers/decoder/mlp/mixture_of_experts.py:243-244). */
+int fm_topk_routing(const void *logits, void *top_experts, void *scores, int64_t num_tokens, int64_t num_experts,
+                    int64_t experts_per_token, int dtype, void *stream);
+
+/* grad_logits[t, top_experts[t, j]] = scores[t, j] * (grad_scores[t, j] - <scores[t, :], grad_scores[t, :]>), zero
+ * elsewhere: what autograd derives for the pair above (same lines of the reference). grad_scores/scores are fp32,
+ * grad_logits has `dtype`. */
+int fm_topk_routing_backward(const void *grad_scores, const void *scores, const void *top_experts, void *grad_logits,
+                             int64_t num_tokens, int64_t num_experts, int64_t experts_per_token, int dtype,
+                             void *stream);
 
 /* ---------------------------------------------------------------------------------------------------------
  * MLP activation. `input` is [num_rows, num_columns * (gated ? 2 : 1)], `output`/`grad_output` are
