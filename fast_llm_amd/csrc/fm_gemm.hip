@@ -188,7 +188,7 @@ extern "C" int fm_output_sparse_matmul(const void *lhs, const void *rhs, void *o
                                        int accumulate, int dtype, int out_dtype, int index_dtype, void *stream) {
     GemmArgs args{lhs, rhs, out, expert_ends, nullptr, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
                   rhs_stride_col, out_stride_row, out_stride_col, row_dim, col_sparse_dim, inner_dim, col_sparse_dim,
-                  static_cast<int>(expert_ends ? num_experts : 1), kOutputSparse, accumulate, index_dtype, out_dtype, 0, 0};
+                  static_cast<int>(expert_ends ? num_experts : 1), kOutputSparse, accumulate, index_dtype, out_dtype, 0, 0, nullptr};
     FM_REQUIRE(num_experts >= 1 && num_experts < (1 << 20), "fm_output_sparse_matmul: bad num_experts");
     return run_gemm("fm_output_sparse_matmul", args, dtype, stream);
 }
@@ -201,7 +201,7 @@ extern "C" int fm_input_inner_sparse_matmul(const void *lhs, const void *rhs, vo
                                             int index_dtype, void *stream) {
     GemmArgs args{lhs, rhs, out, expert_ends, nullptr, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
                   rhs_stride_col, out_stride_row, out_stride_col, row_dim, col_dim, inner_sparse_dim, inner_sparse_dim,
-                  static_cast<int>(expert_ends ? num_experts : 1), kInputInnerSparse, accumulate, index_dtype, out_dtype, 0, 0};
+                  static_cast<int>(expert_ends ? num_experts : 1), kInputInnerSparse, accumulate, index_dtype, out_dtype, 0, 0, nullptr};
     FM_REQUIRE(num_experts >= 1 && num_experts < (1 << 20), "fm_input_inner_sparse_matmul: bad num_experts");
     return run_gemm("fm_input_inner_sparse_matmul", args, dtype, stream);
 }
@@ -216,6 +216,6 @@ extern "C" int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void
     const int64_t experts = expert_ends ? num_experts : 1;
     GemmArgs args{lhs, rhs, out, expert_ends, expert_pad_begins, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
                   rhs_stride_col, out_stride_row, out_stride_col, row_sparse_dim * experts, col_dim, inner_dim,
-                  row_sparse_dim, static_cast<int>(experts), kInputRowSparse, accumulate, index_dtype, out_dtype, 0, 0};
+                  row_sparse_dim, static_cast<int>(experts), kInputRowSparse, accumulate, index_dtype, out_dtype, 0, 0, nullptr};
     return run_gemm("fm_input_row_sparse_matmul", args, dtype, stream);
 }

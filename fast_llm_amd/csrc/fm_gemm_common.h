@@ -24,6 +24,7 @@ struct GemmArgs {
     int index_dtype;
     int out_dtype;
     int tiles_m, tiles_n;
+    float *partials;  // workspace of the MFMA kernel for split reductions, or null; set by its launcher
 };
 
 template <typename OutT>

@@ -32,6 +32,9 @@
 
 #include "fm_gemm_common.h"
 
+#include <mutex>
+#include <stdlib.h>
+
 namespace fm {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
@@ -342,26 +345,122 @@ __device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int tile_m, i
     return true;
 }
 
-// Hardware workgroup id -> (row tile, column tile). The hardware hands consecutive workgroup ids to the 8 XCDs in
-// turn, so the 32 CUs of XCD x run the ids x, x + 8, x + 16, ... in that order. Those are mapped to chunks of 32
-// consecutive logical tiles, chunk c going to XCD c % 8: the tiles an XCD runs at the same time are then one chunk,
-// i.e. 8 row tiles x 4 column tiles that share operand panels in that XCD's L2, while consecutive chunks go to
+// Hardware workgroup id -> position in the logical tile order. The hardware hands consecutive workgroup ids to the
+// 8 XCDs in turn, so the 32 CUs of XCD x run the ids x, x + 8, x + 16, ... in that order. Those are mapped to chunks
+// of 32 consecutive logical tiles, chunk c going to XCD c % 8: the tiles an XCD runs at the same time are then one
+// chunk, i.e. 8 row tiles x 4 column tiles that share operand panels in that XCD's L2, while consecutive chunks go to
 // different XCDs, so that experts with many and with few tokens (long and short tiles of the row-sparse product)
-// are spread over all of them. Returns false for the ids that pad the grid to whole rounds of chunks.
+// are spread over all of them. A permutation of every aligned block of 256 ids.
 constexpr int kXcds = 8, kGroupRows = 8, kChunkTiles = 32;
-__device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int &tile_m, int &tile_n) {
-    const int total = args.tiles_m * args.tiles_n;
-    const int pid = blockIdx.x;
+constexpr int kRound = kXcds * kChunkTiles;  // workgroups that run at the same time: one per CU
+__device__ __forceinline__ int logical_of_block(int pid) {
     const int xcd = pid % kXcds, local = pid / kXcds;
-    const int logical = ((local / kChunkTiles) * kXcds + xcd) * kChunkTiles + local % kChunkTiles;
-    if (logical >= total) return false;
-    const int width = kGroupRows * args.tiles_n;
+    return ((local / kChunkTiles) * kXcds + xcd) * kChunkTiles + local % kChunkTiles;
+}
+
+// Logical tile -> (row tile, column tile): groups of 8 row tiles, column by column inside a group.
+__device__ __forceinline__ void tile_coordinates(int logical, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
+    const int width = kGroupRows * tiles_n;
     const int group = logical / width;
     const int first_m = group * kGroupRows;
-    const int group_rows = min(args.tiles_m - first_m, kGroupRows);
+    const int group_rows = min(tiles_m - first_m, kGroupRows);
     const int in_group = logical - group * width;
     tile_m = first_m + in_group % group_rows;
     tile_n = in_group / group_rows;
+}
+
+// ---- splitting the reduction of the last tiles ---------------------------------------------------------------
+// With T tiles and 256 CUs the launch runs in ceil(T / 256) rounds, and the last one keeps only T % 256 CUs busy: a
+// large loss when there are few, long tiles (4.25 rounds cost 5). When the caller passes a workspace, the tiles of that
+// last round are cut along the reduction axis into `pieces` pieces each, so that they fill the CUs; a piece writes its
+// fp32 accumulators to the workspace and a second kernel adds the pieces of a tile, always in the same order, and
+// stores the result. The plan is a function of the arguments and the expert map only, and every workgroup of both
+// kernels computes the same one.
+constexpr int kMaxPartials = 512;          // workspace slots of 256 x 256 floats
+constexpr int kMinPieceSlices = 16;        // do not cut a reduction into pieces shorter than this
+constexpr int kPieceOverheadSlices = 8;    // set-up, prologue and epilogue of a piece, in slice times
+constexpr int kPartialFloats = kTile * kTile;
+
+struct SplitPlan {
+    int tiles_m;       // row tiles that exist
+    int whole;         // logical tiles [0, whole) are computed by one workgroup each
+    int tail;          // the tiles after them
+    int pieces;        // pieces per tail tile (1: not split)
+    int piece_slices;  // slices per piece (the last piece may have fewer)
+};
+
+// sum over experts of ceil(rows_e / 256). Wave-uniform.
+__device__ __forceinline__ int count_row_tiles(const GemmArgs &args) {
+    if (args.expert_ends == nullptr) return static_cast<int>((args.rows + kTile - 1) / kTile);
+    const int lane = threadIdx.x & 63;
+    int tiles = 0;
+    for (int base = 0; base < args.num_experts; base += 64) {
+        const int e = base + lane;
+        int64_t begin = 0, end = 0;
+        if (e < args.num_experts) {
+            end = min(load_index(args.expert_ends, args.index_dtype, e), args.rows);
+            begin = e > 0 ? load_index(args.expert_ends, args.index_dtype, e - 1) : 0;
+        }
+        int count = end > begin ? static_cast<int>((end - begin + kTile - 1) / kTile) : 0;
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) count += __shfl_xor(count, offset, 64);
+        tiles += count;
+    }
+    return __builtin_amdgcn_readfirstlane(tiles);
+}
+
+__device__ __forceinline__ SplitPlan plan_split(const GemmArgs &args) {
+    SplitPlan plan;
+    plan.tiles_m = count_row_tiles(args);
+    const int total = plan.tiles_m * args.tiles_n;
+    plan.tail = total % kRound;
+    plan.whole = total - plan.tail;
+    plan.pieces = 1;
+    const int num_slices = static_cast<int>(args.inner / kBK);
+    plan.piece_slices = num_slices;
+    int best = num_slices;
+    if (plan.tail > 0) {
+#pragma unroll
+        for (int split = 2; split <= 8; split *= 2) {
+            if (plan.tail * split > kMaxPartials || num_slices / split < kMinPieceSlices) continue;
+            const int length = ((num_slices + split - 1) / split + 1) / 2 * 2;  // even: slices are multiplied in pairs
+            const int pieces = (num_slices + length - 1) / length;
+            const int cost = (plan.tail * pieces + kRound - 1) / kRound * (length + kPieceOverheadSlices);
+            if (cost < best) {
+                best = cost;
+                plan.pieces = pieces;
+                plan.piece_slices = length;
+            }
+        }
+    }
+    return plan;
+}
+
+// What the workgroup `pid` of the main kernel computes. Without a workspace (piece_slot < 0 on return) the row tile
+// count is the host's upper bound and ids past the tiles that exist are weeded out later, by resolve_tile.
+__device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int &tile_m, int &tile_n, int &piece,
+                                              int &piece_slices, int &piece_slot) {
+    int logical = logical_of_block(pid);
+    piece = 0;
+    piece_slices = 0;
+    piece_slot = -1;
+    if (args.partials == nullptr) {
+        if (logical >= args.tiles_m * args.tiles_n) return false;
+        tile_coordinates(logical, args.tiles_m, args.tiles_n, tile_m, tile_n);
+        return true;
+    }
+    const SplitPlan plan = plan_split(args);
+    if (logical >= plan.whole) {
+        const int index = logical - plan.whole;
+        if (index >= plan.tail * plan.pieces) return false;
+        if (plan.pieces > 1) {
+            piece = index / plan.tail;
+            piece_slices = plan.piece_slices;
+            piece_slot = index;
+            logical = plan.whole + index - piece * plan.tail;
+        }
+    }
+    tile_coordinates(logical, plan.tiles_m, args.tiles_n, tile_m, tile_n);
     return true;
 }
 
@@ -436,15 +535,61 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTiles
     }
 }
 
+__device__ __forceinline__ void store_result(const GemmArgs &args, const TileWork &work,
+                                             const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds, int wave,
+                                             int lane) {
+    const bool accumulate = args.accumulate != 0;
+    auto store = [&](auto *out) {
+        if (accumulate)
+            store_tile<std::remove_pointer_t<decltype(out)>, true>(acc, lds, out + work.out_offset, args.out_stride_row,
+                                                                   work.rows_valid, work.cols_valid, wave, lane);
+        else
+            store_tile<std::remove_pointer_t<decltype(out)>, false>(acc, lds, out + work.out_offset, args.out_stride_row,
+                                                                    work.rows_valid, work.cols_valid, wave, lane);
+    };
+    if (args.out_dtype == FM_DTYPE_F32) store(static_cast<float *>(args.out));
+    else if (args.out_dtype == FM_DTYPE_BF16) store(static_cast<bf16_t *>(args.out));
+    else store(static_cast<f16_t *>(args.out));
+}
+
+// A piece's accumulators in the workspace: register by register, 16 bytes per lane, so that every store and load
+// covers 1 KiB of consecutive addresses. [wave][accumulator][group of 4 registers][lane][4]
+template <typename FloatT>
+__device__ __forceinline__ FloatT *partial_of_lane(FloatT *slot, int wave, int lane) {
+    return slot + wave * (kPartialFloats / kWaves) + lane * 4;
+}
+
+__device__ __forceinline__ void store_partial(const f32x16_t (&acc)[kTilesM][kTilesN], float *slot, int wave, int lane) {
+    float *partial = partial_of_lane(slot, wave, lane);
+#pragma unroll
+    for (int i = 0; i < kTilesM; ++i)
+#pragma unroll
+        for (int j = 0; j < kTilesN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4_t value;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) value[c] = acc[i][j][4 * g + c];
+                *reinterpret_cast<f32x4_t *>(partial + ((i * kTilesN + j) * 4 + g) * 256) = value;
+            }
+}
+
 // kMasked: the row-sparse product, whose reduction range [k_lo, k_hi) is ragged.
 template <typename T, bool kLhsContiguousK, bool kRhsContiguousK, bool kMasked>
 __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_kernel(GemmArgs args) {
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);  // C-style: address-space cast
 
-    int tile_m, tile_n;
+    int tile_m, tile_n, piece, piece_slices, piece_slot;
     TileWork work;
-    if (!tile_of_block(args, tile_m, tile_n) || !resolve_tile(args, tile_m, tile_n, work)) return;
+    if (!tile_of_block(args, blockIdx.x, tile_m, tile_n, piece, piece_slices, piece_slot) ||
+        !resolve_tile(args, tile_m, tile_n, work))
+        return;
+    piece_slot = __builtin_amdgcn_readfirstlane(piece_slot);
+    if (piece_slot >= 0) {  // a piece of a tile whose reduction is split (never the row-sparse product)
+        work.k_lo = static_cast<int64_t>(piece) * piece_slices * kBK;
+        work.k_hi = min(work.k_hi, work.k_lo + static_cast<int64_t>(piece_slices) * kBK);
+    }
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -547,7 +692,8 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             }
 #pragma unroll
             for (int m = 0; m < kTilesM * kTilesN; ++m) {
-                const int i = m / kTilesN, j = m % kTilesN;
+                // Boustrophedon order: consecutive MFMAs always share one operand (fewer operand-bus toggles).
+                const int i = m / kTilesN, j = (i & 1) ? kTilesN - 1 - m % kTilesN : m % kTilesN;
                 acc[i][j] = Mfma<T>::run(frag_b[buffer][j], frag_a[buffer][i], acc[i][j]);  // transposed, see store_tile
                 if (m < 4) {
                     read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
@@ -611,37 +757,80 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         wait_for_loads<0>();  // the zero-filling loads of slices past the end still write LDS
     }
 
-    const bool accumulate = args.accumulate != 0;
-    if (accumulate && num_slices == 0) return;  // nothing to add
+    if (piece_slot < 0 && args.accumulate != 0 && num_slices == 0) return;  // nothing to add
     __syncthreads();  // all wavefronts are done reading operand slices; LDS becomes the staging area
-    auto store = [&](auto *out) {
-        if (accumulate)
-            store_tile<std::remove_pointer_t<decltype(out)>, true>(acc, lds, out + work.out_offset, args.out_stride_row,
-                                                                   work.rows_valid, work.cols_valid, wave, lane);
-        else
-            store_tile<std::remove_pointer_t<decltype(out)>, false>(acc, lds, out + work.out_offset, args.out_stride_row,
-                                                                    work.rows_valid, work.cols_valid, wave, lane);
-    };
-    if (args.out_dtype == FM_DTYPE_F32) store(static_cast<float *>(args.out));
-    else if (args.out_dtype == FM_DTYPE_BF16) store(static_cast<bf16_t *>(args.out));
-    else store(static_cast<f16_t *>(args.out));
+    if (piece_slot >= 0) store_partial(acc, args.partials + static_cast<int64_t>(piece_slot) * kPartialFloats, wave, lane);
+    else store_result(args, work, acc, lds, wave, lane);
+}
+
+// Adds the pieces of each tile whose reduction the main kernel split, in piece order, and stores the sums.
+// One workgroup per tile of the last round.
+__global__ __launch_bounds__(kMfmaThreads) void grouped_gemm_reduce_kernel(GemmArgs args) {
+    extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
+    FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);
+    const SplitPlan plan = plan_split(args);
+    const int index = blockIdx.x;
+    if (plan.pieces == 1 || index >= plan.tail) return;
+    int tile_m, tile_n;
+    TileWork work;
+    tile_coordinates(plan.whole + index, plan.tiles_m, args.tiles_n, tile_m, tile_n);
+    if (!resolve_tile(args, tile_m, tile_n, work)) return;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    f32x16_t acc[kTilesM][kTilesN];
+#pragma unroll
+    for (int i = 0; i < kTilesM; ++i)
+#pragma unroll
+        for (int j = 0; j < kTilesN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    for (int piece = 0; piece < plan.pieces; ++piece) {
+        const float *partial = partial_of_lane(
+            args.partials + static_cast<int64_t>(piece * plan.tail + index) * kPartialFloats, wave, lane);
+#pragma unroll
+        for (int i = 0; i < kTilesM; ++i)
+#pragma unroll
+            for (int j = 0; j < kTilesN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4_t value =
+                        *reinterpret_cast<const f32x4_t *>(partial + ((i * kTilesN + j) * 4 + g) * 256);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        acc[i][j][4 * g + c] += value[c];
+                }
+    }
+    store_result(args, work, acc, lds, wave, lane);
 }
 
 // ---- host side -----------------------------------------------------------------------------------------
+static int allow_big_lds(const void *kernel) {
+    hipError_t error = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
+    return FM_OK;
+}
+
 template <typename T, bool kLhsK, bool kRhsK, bool kMasked>
 static int launch_instance(const GemmArgs &args, hipStream_t stream) {
     auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK, kMasked>;
     static bool configured = false;  // setting the attribute twice from racing threads is harmless
     if (!configured) {
-        hipError_t error = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-        if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
+        if (int status = allow_big_lds(reinterpret_cast<const void *>(kernel))) return status;
         configured = true;
     }
-    // Whole rounds of one chunk per XCD; the surplus workgroups find no tile and exit.
-    constexpr int kRound = kXcds * kChunkTiles;
-    const int grid = (args.tiles_m * args.tiles_n + kRound - 1) / kRound * kRound;
+    // Whole rounds of one chunk per XCD; the surplus workgroups find no tile and exit. With a workspace the pieces
+    // of the last round's tiles come after the whole tiles, at most kMaxPartials of them.
+    int grid = (args.tiles_m * args.tiles_n + kRound - 1) / kRound * kRound;
+    if (args.partials != nullptr) grid += kMaxPartials;
     kernel<<<grid, kMfmaThreads, kLdsBytes, stream>>>(args);
+    if (args.partials != nullptr) {
+        static bool reduce_configured = false;
+        if (!reduce_configured) {
+            if (int status = allow_big_lds(reinterpret_cast<const void *>(grouped_gemm_reduce_kernel))) return status;
+            reduce_configured = true;
+        }
+        grouped_gemm_reduce_kernel<<<kRound, kMfmaThreads, kLdsBytes, stream>>>(args);
+    }
     return FM_OK;
 }
 
@@ -681,6 +870,53 @@ bool mfma_gemm_eligible(const GemmArgs &args, int dtype) {
     return true;
 }
 
+// ---- workspace for split reductions --------------------------------------------------------------------
+// kMaxPartials tiles of fp32 (128 MiB) per (device, stream) that has needed one, allocated at the first such call and
+// kept until the process ends. Kernels on one stream run in order, so calls on one stream can share a workspace;
+// calls on different streams may overlap and get their own.
+namespace {
+struct Workspace {
+    int device;
+    hipStream_t stream;
+    float *pointer;
+};
+constexpr int kMaxWorkspaces = 16;
+Workspace workspaces[kMaxWorkspaces];
+int num_workspaces = 0;
+std::mutex workspace_mutex;
+
+bool split_enabled() {
+    static const bool enabled = [] {
+        const char *value = getenv("FASTMOE_SPLIT_REDUCTION");
+        return value == nullptr || value[0] != '0';
+    }();
+    return enabled;
+}
+
+// Null when there is none and none can be had (table full, out of memory, stream under graph capture): the product
+// then runs without splitting.
+float *split_workspace(hipStream_t stream) {
+    int device;
+    if (hipGetDevice(&device) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(workspace_mutex);
+    for (int i = 0; i < num_workspaces; ++i)
+        if (workspaces[i].device == device && workspaces[i].stream == stream) return workspaces[i].pointer;
+    if (num_workspaces == kMaxWorkspaces) return nullptr;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    void *pointer = nullptr;
+    if (hipMalloc(&pointer, sizeof(float) * kPartialFloats * kMaxPartials) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    workspaces[num_workspaces++] = {device, stream, static_cast<float *>(pointer)};
+    return static_cast<float *>(pointer);
+}
+}  // namespace
+
 int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream) {
     if (args.mode == kInputRowSparse) {
         args.tiles_m = static_cast<int>((args.sparse_size + kTile - 1) / kTile) * args.num_experts;
@@ -689,8 +925,14 @@ int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream) {
         args.tiles_m = static_cast<int>((args.rows + kTile - 1) / kTile + (args.expert_ends ? args.num_experts : 0));
     }
     args.tiles_n = static_cast<int>((args.cols + kTile - 1) / kTile);
-    if (static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31) - 256)
+    if (static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31) - 1024)
         return fail(FM_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
+    // Splitting the last round's reductions can pay when the rounds are few and the reduction is long.
+    args.partials = nullptr;
+    constexpr int kMaxRoundsToSplit = 16;
+    if (args.mode != kInputRowSparse && args.inner / kBK >= 2 * kMinPieceSlices &&
+        static_cast<int64_t>(args.tiles_m) * args.tiles_n <= kMaxRoundsToSplit * kRound && split_enabled())
+        args.partials = split_workspace(stream);
     return dtype == FM_DTYPE_BF16 ? launch_layout<bf16_t>(args, stream) : launch_layout<f16_t>(args, stream);
 }
 

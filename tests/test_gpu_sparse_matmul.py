@@ -302,3 +302,45 @@ def test_mfma_kernel_on_ragged_experts(experts, dense_dim, sparse_dim, dtype, de
         assert max_rel_err(out.cpu(), expected) <= tolerance
         input_row_sparse_matmul(y_poisoned.t(), x_poisoned, sparse_map, out=out, accumulate=True)
         assert max_rel_err(out.cpu(), 2 * expected.float()) <= tolerance
+
+
+# Few tiles and a long reduction: the tiles of the last round of workgroups are cut along the reduction axis and their
+# pieces added by a second kernel. (experts, reduction size, other size): 4 pieces of 18 slices with a shorter, odd last
+# one; whole tiles followed by more than 256 pieces; 2 pieces.
+@pytest.mark.parametrize(("experts", "inner", "other"), [(9, 4160, 320), (70, 2240, 600), (40, 4096, 256), (3, 2048, 264)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_split_reduction_of_last_round(experts, inner, other, dtype, device):
+    case = _ragged_case(experts + inner, experts)
+    oracle_map = fixture_sparse_map(case)
+    oracle_map.num_rows = case["expert_ends"][-1] + case["phantom_rows"]
+    sparse_map = to_device_map(oracle_map, device, torch.int32)
+    used = _used_rows(oracle_map)
+    generator = torch.Generator().manual_seed(13)
+    tolerance = _MAX_REL[dtype]
+
+    # output-sparse: [rows, inner] x per-expert [inner, other]
+    x, weight = _normal(oracle_map.num_rows, inner, dtype, generator), _normal(experts * other, inner, dtype, generator)
+    x_gpu, weight_gpu = x.to(device), weight.to(device)
+    expected = moe_oracle.output_sparse_matmul(x, weight.t(), oracle_map)
+    out = torch.full((oracle_map.num_rows, other), 5.0, dtype=dtype, device=device)
+    output_sparse_matmul(x_gpu, weight_gpu.t(), sparse_map, out)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+    assert (out[used:] == 5.0).all()
+    again = torch.empty_like(out)
+    output_sparse_matmul(x_gpu, weight_gpu.t(), sparse_map, again)
+    assert torch.equal(out[:used], again[:used])
+    # accumulation into a wider output
+    previous = _normal(oracle_map.num_rows, other, torch.float32, generator)
+    out = previous.to(device)
+    output_sparse_matmul(x_gpu, weight_gpu.t(), sparse_map, out, accumulate=True)
+    assert max_rel_err(out[:used].cpu(), (expected.float() + previous)[:used]) <= tolerance
+    assert torch.equal(out[used:].cpu(), previous[used:])
+
+    # input-inner-sparse: [rows, inner] x per-expert [inner, other], weight stored [experts * inner, other]
+    weight = _normal(experts * inner, other, dtype, generator)
+    out = input_inner_sparse_matmul(x_gpu, weight.to(device), sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(x, weight, oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+    # dense product through the same kernel
+    expected = (x.float() @ weight[:inner].float()).to(dtype)
+    assert max_rel_err(dense_matmul(x_gpu, weight[:inner].to(device)).cpu(), expected) <= tolerance
