@@ -77,3 +77,112 @@ def topk_routing(logits: torch.Tensor, experts_per_token: int) -> tuple[torch.Te
     scores, top_experts = _TopKRouting.apply(flat, experts_per_token)
     shape = logits.shape[:-1] + (experts_per_token,)
     return scores.view(shape), top_experts.view(shape)
+
+
+def router_forward(
+    logits: torch.Tensor, noise: torch.Tensor | None, experts_per_token: int, shared_experts: int
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One pass over `logits` [tokens, routed experts]: (scores fp32, top_experts int64, both
+    [tokens, shared_experts + k]; losses [2] fp32 = load-balancing loss, z-loss; and lse [tokens, 2], statistics
+    [2 * experts + 1], both kept for the backward)."""
+    assert logits.dim() == 2 and logits.is_contiguous()
+    assert noise is None or (noise.shape == logits.shape and noise.dtype == logits.dtype and noise.is_contiguous())
+    device = _lib.require_device(logits, noise)
+    tokens, experts = logits.shape
+    if not 0 < experts_per_token <= experts:
+        raise ValueError(f"experts_per_token={experts_per_token} with {experts} experts")
+    if tokens == 0:
+        raise ValueError("no tokens to route")
+    slots = shared_experts + experts_per_token
+    new = lambda shape, dtype: torch.empty(shape, dtype=dtype, device=logits.device)  # noqa: E731
+    scores, top_experts = new((tokens, slots), torch.float32), new((tokens, slots), torch.int64)
+    lse, statistics, losses = new((tokens, 2), torch.float32), new(2 * experts + 1, torch.float32), new(2, torch.float32)
+    workspace_size = _lib.lib().fm_router_workspace_size(tokens, experts)
+    workspace = new(workspace_size, torch.uint8)
+    _lib.call(
+        "fm_router_forward",
+        device,
+        _lib.ptr(logits),
+        _lib.ptr(noise),
+        _lib.ptr(top_experts),
+        _lib.ptr(scores),
+        _lib.ptr(lse),
+        _lib.ptr(statistics),
+        _lib.ptr(losses),
+        _lib.ptr(workspace),
+        workspace_size,
+        tokens,
+        experts,
+        experts_per_token,
+        shared_experts,
+        _lib.dtype_tag(logits.dtype),
+    )
+    return scores, top_experts, losses, lse, statistics
+
+
+class _Router(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, noise, experts_per_token, shared_experts, auxiliary_loss_grad, z_loss_grad):
+        logits = logits.detach().contiguous()
+        noise = None if noise is None else noise.detach().contiguous()
+        scores, top_experts, losses, lse, statistics = router_forward(logits, noise, experts_per_token, shared_experts)
+        ctx.save_for_backward(logits, noise, scores, top_experts, lse, statistics)
+        ctx.shape = (experts_per_token, shared_experts)
+        ctx.loss_grads = (auxiliary_loss_grad or 0.0, z_loss_grad or 0.0)
+        ctx.mark_non_differentiable(top_experts, losses)
+        return scores, top_experts, losses
+
+    @staticmethod
+    def backward(ctx, grad_scores, _, __):
+        logits, noise, scores, top_experts, lse, statistics = ctx.saved_tensors
+        experts_per_token, shared_experts = ctx.shape
+        device = _lib.require_device(logits)
+        grad_logits = torch.empty_like(logits)
+        _lib.call(
+            "fm_router_backward",
+            device,
+            _lib.ptr(grad_scores.to(torch.float32).contiguous()),
+            _lib.ptr(scores),
+            _lib.ptr(top_experts),
+            _lib.ptr(logits),
+            _lib.ptr(noise),
+            _lib.ptr(lse),
+            _lib.ptr(statistics),
+            _lib.ptr(grad_logits),
+            float(ctx.loss_grads[0]),
+            float(ctx.loss_grads[1]),
+            logits.size(0),
+            logits.size(1),
+            experts_per_token,
+            shared_experts,
+            _lib.dtype_tag(logits.dtype),
+        )
+        return grad_logits, None, None, None, None, None
+
+
+def router(
+    logits: torch.Tensor,
+    experts_per_token: int,
+    *,
+    shared_experts: int = 0,
+    noise: torch.Tensor | None = None,
+    auxiliary_loss_grad: float | None = None,
+    z_loss_grad: float | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """
+    The router front end of `MixtureOfExpertMLP._forward` for top-k routing (reference:
+    fast_llm/layers/decoder/mlp/mixture_of_experts.py:146-171, 237-278) in one pass over `logits` [..., routed experts]:
+    z-loss, jitter (`noise`, the multiplier the caller drew), top-k + fp32 softmax, load-balancing loss, shared experts.
+    Returns (scores [..., shared + k] fp32, top_experts int64, load_balancing_loss, z_loss); the two losses are
+    detached scalars. `auxiliary_loss_grad` / `z_loss_grad` are the constant gradients the reference's `AuxiliaryLoss`
+    (functional/utils.py:63-71) gives the losses when the scores are back-propagated:
+    `unshared_experts * auxiliary_loss_coefficient * grad_scale` and `z_loss_coefficient * grad_scale`; None or 0:
+    that loss contributes no gradient.
+    """
+    flat = logits.flatten(0, -2)
+    flat_noise = None if noise is None else noise.flatten(0, -2)
+    scores, top_experts, losses = _Router.apply(
+        flat, flat_noise, experts_per_token, shared_experts, auxiliary_loss_grad, z_loss_grad
+    )
+    shape = logits.shape[:-1] + (shared_experts + experts_per_token,)
+    return scores.view(shape), top_experts.view(shape), losses[0], losses[1]

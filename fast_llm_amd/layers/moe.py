@@ -2,10 +2,10 @@
 A single-GPU dropless mixture-of-experts MLP block built on the HIP kernel path.
 
 Covers what `MixtureOfExpertMLP` does between the router input and the block output for top-k routing
-(reference: fast_llm/layers/decoder/mlp/mixture_of_experts.py:130-213, 237-262): router logits, top-k experts, fp32
-softmax over the selected logits, sparse map, dropless MLP. Weight layout as in the reference: `layer_1.weight`
-[experts * 2 * ffn, hidden] with each expert's block ordered [gate; up] (layers/decoder/mlp/mlp.py:81-87),
-`layer_2.weight` [experts * ffn, hidden] (stored transposed, :70-79).
+(reference: fast_llm/layers/decoder/mlp/mixture_of_experts.py:130-213, 237-278): router logits, z-loss, jitter, top-k
+experts, fp32 softmax over the selected logits, load-balancing loss, shared experts, sparse map, dropless MLP.
+Weight layout as in the reference: `layer_1.weight` [experts * 2 * ffn, hidden] with each expert's block ordered
+[gate; up] (layers/decoder/mlp/mlp.py:81-87), `layer_2.weight` [experts * ffn, hidden] (stored transposed, :70-79).
 """
 
 import torch
@@ -23,7 +23,9 @@ def attach_grad_buffer(weight: torch.Tensor, dtype: torch.dtype | None = None) -
     return weight
 
 
-from fast_llm_amd.functional.routing import topk_routing  # noqa: E402  (re-exported: the layer's routing step)
+from fast_llm_amd.functional.routing import router, topk_routing  # noqa: E402, F401  (re-exported)
+
+LOAD_BALANCING_LOSS, ROUTER_Z_LOSS = "load_balancing_loss", "router_z_loss"  # layers/decoder/mlp/config.py:24-26
 
 
 class DroplessMoEMLP(torch.nn.Module):
@@ -38,17 +40,28 @@ class DroplessMoEMLP(torch.nn.Module):
         activation: ActivationType = ActivationType.silu,
         recompute_level: MLPRecomputeLevel = MLPRecomputeLevel.none,
         dropless_dynamic_shape: bool = False,
+        shared_experts: int = 0,
+        auxiliary_loss_coefficient: float = 0.01,
+        z_loss_coefficient: float = 0.0,
+        jitter_eps: float = 0.0,
         full_precision_gradients: bool = False,
         init_std: float = 0.02,
         dtype: torch.dtype = torch.bfloat16,
         device: torch.device | str = "cuda",
     ):
         super().__init__()
-        self.experts, self.experts_per_token = experts, experts_per_token
+        # `experts` counts the shared experts, which every token visits on top of its `experts_per_token` routed ones
+        # (layers/decoder/mlp/config.py:127-133, 181-187).
+        if not 0 <= shared_experts <= experts - experts_per_token:
+            raise ValueError(f"shared_experts={shared_experts} with {experts} experts, {experts_per_token} per token")
+        self.experts, self.experts_per_token, self.shared_experts = experts, experts_per_token, shared_experts
+        self.unshared_experts = experts - shared_experts
+        self.auxiliary_loss_coefficient, self.z_loss_coefficient = auxiliary_loss_coefficient, z_loss_coefficient
+        self.jitter_eps = jitter_eps
         self.gated, self.activation = gated, activation
         self.recompute_level, self.dropless_dynamic_shape = recompute_level, dropless_dynamic_shape
         layer_1_rows = experts * intermediate_size * (2 if gated else 1)
-        self.router = torch.nn.Parameter(torch.empty(experts, hidden_size, dtype=dtype, device=device))
+        self.router = torch.nn.Parameter(torch.empty(self.unshared_experts, hidden_size, dtype=dtype, device=device))
         self.layer_1 = torch.nn.Parameter(torch.empty(layer_1_rows, hidden_size, dtype=dtype, device=device))
         self.layer_2 = torch.nn.Parameter(
             torch.empty(experts * intermediate_size, hidden_size, dtype=dtype, device=device)
@@ -60,20 +73,44 @@ class DroplessMoEMLP(torch.nn.Module):
         attach_grad_buffer(self.layer_1, grad_dtype)
         attach_grad_buffer(self.layer_2, grad_dtype)
 
-    def route(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    def route(
+        self, hidden_states: torch.Tensor, grad_scale: float | None = None, losses: dict | None = None
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """Router logits to (scores, top_experts), shared experts included. `grad_scale` (the reference's
+        `kwargs["grad_output"]`) makes the two auxiliary losses train the router; `losses` collects their values
+        (mixture_of_experts.py:146-171, 237-262)."""
         logits = torch.nn.functional.linear(hidden_states, self.router)
-        return topk_routing(logits, self.experts_per_token)
+        noise = None
+        if self.training and self.jitter_eps > 0.0:
+            noise = torch.empty_like(logits).uniform_(1.0 - self.jitter_eps, 1.0 + self.jitter_eps)
+        trained = self.training and grad_scale is not None
+        scores, top_experts, load_balancing_loss, z_loss = router(
+            logits,
+            self.experts_per_token,
+            shared_experts=self.shared_experts,
+            noise=noise,
+            auxiliary_loss_grad=self.unshared_experts * self.auxiliary_loss_coefficient * grad_scale if trained else None,
+            z_loss_grad=self.z_loss_coefficient * grad_scale if trained else None,
+        )
+        if losses is not None:
+            losses.setdefault(LOAD_BALANCING_LOSS, []).append(load_balancing_loss)
+            if self.z_loss_coefficient > 0.0:
+                losses.setdefault(ROUTER_Z_LOSS, []).append(z_loss)
+        return scores, top_experts
 
     def forward(
         self,
         input_: torch.Tensor,
         scores: torch.Tensor | None = None,
         top_experts: torch.Tensor | None = None,
+        *,
+        grad_scale: float | None = None,
+        losses: dict | None = None,
     ) -> torch.Tensor:
         """`scores`/`top_experts` may be passed to bypass the router (tests pin the routing that way)."""
         hidden_states = input_.flatten(0, -2)
         if top_experts is None:
-            scores, top_experts = self.route(hidden_states)
+            scores, top_experts = self.route(hidden_states, grad_scale, losses)
         sparse_map = get_sparse_map(top_experts, self.experts, dynamic_shape=self.dropless_dynamic_shape)
         output = mlp_autograd(
             hidden_states,

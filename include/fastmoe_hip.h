@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 2
+#define FM_VERSION 3
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -143,6 +143,35 @@ int fm_topk_routing(const void *logits, void *top_experts, void *scores, int64_t
 int fm_topk_routing_backward(const void *grad_scores, const void *scores, const void *top_experts, void *grad_logits,
                              int64_t num_tokens, int64_t num_experts, int64_t experts_per_token, int dtype,
                              void *stream);
+
+/* The whole router front end of `MixtureOfExpertMLP._forward` between the logits and the sparse map, from one read
+ * of the logits [num_tokens, num_experts] (`dtype`), where num_experts counts the routed (unshared) experts:
+ *   - z-loss = mean_t logsumexp(logits[t, :])^2 on the logits as given
+ *     (fast_llm/layers/decoder/mlp/mixture_of_experts.py:147-154, layers/language_model/loss/z_loss.py:88-92);
+ *   - jitter: if `noise` (same shape and dtype, drawn by the caller) is not null, routing uses logits * noise rounded
+ *     to `dtype` (:157-159, 234-235);
+ *   - top-k and fp32 softmax over the selected logits (:243-244), as fm_topk_routing;
+ *   - load-balancing loss = sum_e mean_t softmax(routed logits)[t, e] * mean_t selected[t, e] (:245-254);
+ *   - shared experts (:264-278): top_experts/scores are [num_tokens, shared_experts + experts_per_token]; the first
+ *     shared_experts slots of every token hold experts num_experts, num_experts + 1, ... with score 1.
+ * Outputs: top_experts (int64), scores (fp32), lse [num_tokens, 2] fp32 (logsumexp of the routed and of the given
+ * logits; kept for the backward), statistics [2 * num_experts + 1] fp32 (per expert: sum_t softmax, number of tokens
+ * that selected it; then sum_t logsumexp^2), losses [2] fp32 (load balancing, z). Sums over tokens are added in a
+ * fixed order. `workspace`: fm_router_workspace_size(num_tokens, num_experts) bytes of device memory. */
+size_t fm_router_workspace_size(int64_t num_tokens, int64_t num_experts);
+int fm_router_forward(const void *logits, const void *noise, void *top_experts, void *scores, void *lse,
+                      void *statistics, void *losses, void *workspace, size_t workspace_size, int64_t num_tokens,
+                      int64_t num_experts, int64_t experts_per_token, int64_t shared_experts, int dtype, void *stream);
+
+/* Gradient of the logits given grad_scores [num_tokens, shared_experts + experts_per_token] (fp32; the shared slots
+ * are ignored) and the constant gradients the reference attaches to the two losses through `AuxiliaryLoss`
+ * (fast_llm/functional/utils.py:63-71; mixture_of_experts.py:154, 257-261): auxiliary_loss_grad for the load-balancing
+ * loss and z_loss_grad for the z-loss, 0 for a loss that is not trained on. logits, noise, scores, top_experts, lse
+ * and statistics are the forward's. grad_logits has `dtype`. */
+int fm_router_backward(const void *grad_scores, const void *scores, const void *top_experts, const void *logits,
+                       const void *noise, const void *lse, const void *statistics, void *grad_logits,
+                       double auxiliary_loss_grad, double z_loss_grad, int64_t num_tokens, int64_t num_experts,
+                       int64_t experts_per_token, int64_t shared_experts, int dtype, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------------
  * MLP activation. `input` is [num_rows, num_columns * (gated ? 2 : 1)], `output`/`grad_output` are

@@ -21,6 +21,8 @@ fast_llm/functional/config.py:31), so the restatement is pinned instead by indep
 | mlp_activation_forward/backward       | torch autograd of `act(x1) * x2` in float64                                            |
 | mlp_forward / mlp_backward (dropless) | the per-expert looped MoE with torch autograd in float64, padding rows NaN-poisoned   |
 | looped_moe                            | a per-token double loop (textbook top-k mixture) in float64                            |
+| router / router_backward              | closed forms (uniform and collapsed routers), a per-token loop in Python floats,       |
+|                                       | central differences of the trained objective (tests/test_oracle_router.py)             |
 
 Arithmetic convention of the oracle: every product and sum is evaluated in `compute_dtype` (float32 by default,
 float64 for pinning), and every tensor the kernels would store is rounded once to the storage dtype of its inputs.
@@ -444,3 +446,60 @@ def topk_routing(logits: torch.Tensor, experts_per_token: int) -> tuple[torch.Te
     (fast_llm/layers/decoder/mlp/mixture_of_experts.py:243-244)."""
     top_logits, top_experts = torch.topk(logits, k=experts_per_token, dim=-1)
     return torch.softmax(top_logits, dim=-1, dtype=torch.float32), top_experts
+
+
+@dataclasses.dataclass
+class RouterResult:
+    scores: torch.Tensor  # [tokens, shared + k] fp32
+    top_experts: torch.Tensor  # [tokens, shared + k] int64
+    load_balancing_loss: torch.Tensor  # scalar fp32
+    z_loss: torch.Tensor  # scalar fp32
+
+
+def router(
+    logits: torch.Tensor,
+    experts_per_token: int,
+    shared_experts: int = 0,
+    noise: torch.Tensor | None = None,
+    compute_dtype: torch.dtype = torch.float32,
+) -> RouterResult:
+    """What `MixtureOfExpertMLP._forward` does between the router's logits and the sparse map, for top-k routing
+    (fast_llm/layers/decoder/mlp/mixture_of_experts.py:146-171), differentiable with torch autograd as there:
+    z-loss on the logits as they come (:147-154; layers/language_model/loss/z_loss.py:88-92), jitter (:157-159,
+    234-235: a product in the logits' own dtype), `_topk_routing` with its load-balancing loss (:243-254), then
+    `_add_shared_experts` (:264-278). `logits` has one column per routed expert. The softmaxes run in
+    `compute_dtype` (the reference's float32; float64 for pinning)."""
+    z_loss = (torch.logsumexp(logits.to(compute_dtype), dim=-1) ** 2).mean()
+    if noise is not None:
+        logits = logits * noise
+    top_logits, top_experts = torch.topk(logits, k=experts_per_token, dim=-1)
+    scores = torch.softmax(top_logits, dim=-1, dtype=compute_dtype)
+    probabilities = torch.softmax(logits, dim=-1, dtype=compute_dtype)
+    mask = torch.nn.functional.one_hot(top_experts, num_classes=logits.size(-1)).sum(dim=1)
+    load_balancing_loss = torch.sum(probabilities.mean(dim=0) * mask.mean(dim=0, dtype=compute_dtype))
+    if shared_experts > 0:
+        first = logits.size(-1)
+        shared = torch.arange(first, first + shared_experts, dtype=top_experts.dtype)[None].repeat(logits.size(0), 1)
+        top_experts = torch.cat((shared, top_experts), dim=1)
+        scores = torch.cat((scores.new_ones(scores.size(0), shared_experts), scores), dim=1)
+    return RouterResult(scores, top_experts, load_balancing_loss, z_loss)
+
+
+def router_backward(
+    result: RouterResult,
+    logits: torch.Tensor,
+    grad_scores: torch.Tensor,
+    auxiliary_loss_grad: float = 0.0,
+    z_loss_grad: float = 0.0,
+) -> torch.Tensor:
+    """Gradient of `logits` (a leaf that `result` was computed from). `AuxiliaryLoss` hands each loss a constant
+    gradient when the scores (or logits) it is attached to are back-propagated (fast_llm/functional/utils.py:63-71):
+    `unshared_experts * auxiliary_loss_coefficient * grad_scale` for the load-balancing loss
+    (mixture_of_experts.py:257-261) and `z_loss_coefficient * grad_scale` for the z-loss (:154)."""
+    total = (
+        (result.scores * grad_scores.to(result.scores.dtype)).sum()
+        + auxiliary_loss_grad * result.load_balancing_loss
+        + z_loss_grad * result.z_loss
+    )
+    (grad_logits,) = torch.autograd.grad(total, logits)
+    return grad_logits

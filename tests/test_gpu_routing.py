@@ -4,7 +4,7 @@ fast_llm/layers/decoder/mlp/mixture_of_experts.py:243-244) and against autograd 
 import pytest
 import torch
 
-from fast_llm_amd.functional.routing import topk_routing
+from fast_llm_amd.functional.routing import router, topk_routing
 from oracle import moe_oracle
 
 pytestmark = pytest.mark.gpu
@@ -70,6 +70,92 @@ def test_topk_routing_backward(tokens, experts, k, dtype, device):
     assert (gpu_logits.grad.cpu()[~selected] == 0).all()
 
 
+def _spaced_logits(tokens, experts, dtype, generator):
+    """Rows that stay free of ties after a jitter of a few percent, also in half precision: a random permutation of
+    1, 1.25, 1.5, ... (exact in bf16 up to 64 experts), plus a small perturbation in fp32."""
+    values = 1 + 0.25 * torch.arange(experts, dtype=torch.float32)
+    order = torch.rand(tokens, experts, generator=generator).argsort(dim=-1)
+    logits = values[order]
+    if dtype == torch.float32:
+        logits = logits + 0.05 * torch.randn(tokens, experts, generator=generator)
+    return logits.to(dtype)
+
+
+# (tokens, experts, k, shared experts, jitter): the benchmark's routers, a token count that leaves workgroups of the
+# forward kernel with unequal or no share, more experts than a wavefront has lanes.
+_ROUTER_CASES = [
+    (8192, 8, 2, 0, False),
+    (2048, 8, 2, 1, True),
+    (1000, 64, 6, 2, False),
+    (16411, 8, 2, 0, True),
+    (37, 8, 3, 0, False),
+    (300, 130, 8, 3, False),
+    (5, 1000, 60, 4, False),
+    (1, 2, 1, 0, True),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(("tokens", "experts", "k", "shared", "jitter"), _ROUTER_CASES)
+def test_router_forward_and_backward(tokens, experts, k, shared, jitter, dtype, device):
+    generator = torch.Generator().manual_seed(tokens + experts)
+    if jitter:
+        logits = _spaced_logits(tokens, experts, dtype, generator)
+        noise = torch.empty(tokens, experts).uniform_(0.99, 1.01, generator=generator).to(dtype)
+    else:
+        logits, noise = _distinct_logits(tokens, experts, dtype, generator), None
+    grad_scores = torch.randn(tokens, shared + k, generator=generator)
+    auxiliary_loss_grad, z_loss_grad = 0.01 * experts * tokens, 0.001 * tokens
+
+    # The oracle in the reference's arithmetic: the jitter product in `dtype`, softmaxes in fp32.
+    leaf = logits.clone().requires_grad_()
+    expected = moe_oracle.router(leaf, k, shared, noise)
+    expected_grad = moe_oracle.router_backward(expected, leaf, grad_scores, auxiliary_loss_grad, z_loss_grad)
+
+    gpu_logits = logits.to(device).requires_grad_()
+    scores, top_experts, load_balancing_loss, z_loss = router(
+        gpu_logits,
+        k,
+        shared_experts=shared,
+        noise=None if noise is None else noise.to(device),
+        auxiliary_loss_grad=auxiliary_loss_grad,
+        z_loss_grad=z_loss_grad,
+    )
+    assert scores.dtype == torch.float32 and top_experts.dtype == torch.int64
+    assert not load_balancing_loss.requires_grad and not z_loss.requires_grad
+    assert torch.equal(top_experts.cpu(), expected.top_experts)
+    assert torch.allclose(scores.cpu(), expected.scores.detach(), rtol=2e-6, atol=1e-7)
+    assert load_balancing_loss.item() == pytest.approx(expected.load_balancing_loss.item(), rel=1e-5)
+    assert z_loss.item() == pytest.approx(expected.z_loss.item(), rel=1e-5)
+
+    scores.backward(grad_scores.to(device))
+    assert gpu_logits.grad.dtype == dtype
+    tolerance = 1e-5 if dtype == torch.float32 else 1e-2
+    error = (gpu_logits.grad.float().cpu() - expected_grad.float()).abs().max().item()
+    assert error <= tolerance * expected_grad.float().abs().max().item()
+
+
+def test_router_without_trained_losses_matches_plain_topk_routing(device):
+    generator = torch.Generator().manual_seed(2)
+    logits = torch.randn(777, 16, generator=generator).to(device)
+    grad_scores = torch.randn(777, 4, generator=generator).to(device)
+    plain_logits, fused_logits = logits.clone().requires_grad_(), logits.clone().requires_grad_()
+    plain_scores, plain_experts = topk_routing(plain_logits, 4)
+    fused_scores, fused_experts, _, _ = router(fused_logits, 4)
+    assert torch.equal(plain_experts, fused_experts) and torch.equal(plain_scores, fused_scores)
+    plain_scores.backward(grad_scores)
+    fused_scores.backward(grad_scores)
+    assert torch.equal(plain_logits.grad, fused_logits.grad)
+
+
+def test_router_statistics_do_not_depend_on_scheduling(device):
+    logits = torch.randn(30000, 64, generator=torch.Generator().manual_seed(4)).to(device)
+    first = router(logits, 6)
+    for _ in range(3):
+        again = router(logits, 6)
+        assert all(torch.equal(a, b) for a, b in zip(first, again))
+
+
 def test_routing_feeds_the_layer(device):
     """The layer's router path uses the kernel and stays differentiable down to the router weights."""
     from fast_llm_amd.layers.moe import DroplessMoEMLP
@@ -81,3 +167,43 @@ def test_routing_feeds_the_layer(device):
     out.float().square().mean().backward()
     assert torch.isfinite(out).all() and x.grad is not None and layer.router.grad is not None
     assert layer.router.grad.abs().sum() > 0
+
+
+def test_layer_with_shared_experts_and_trained_router_losses(device):
+    """The whole block, router included, against the oracle's router followed by its per-expert loop, with torch
+    autograd of both for the gradients down to the router weights."""
+    from fast_llm_amd.layers.moe import LOAD_BALANCING_LOSS, ROUTER_Z_LOSS, DroplessMoEMLP
+
+    torch.manual_seed(1)
+    tokens, hidden, ffn, experts, k, shared = 384, 128, 128, 6, 2, 1
+    coefficient, z_coefficient, grad_scale = 0.05, 0.002, 3.0
+    layer = DroplessMoEMLP(
+        hidden, ffn, experts, k, shared_experts=shared, auxiliary_loss_coefficient=coefficient,
+        z_loss_coefficient=z_coefficient, init_std=0.1, dtype=torch.float32, device=device,
+    )  # fmt: skip
+    x = torch.randn(tokens, hidden, device=device, requires_grad=True)
+    grad_output = torch.randn(tokens, hidden, device=device)
+    losses = {}
+    out = layer(x, grad_scale=grad_scale, losses=losses)
+    out.backward(grad_output)
+
+    leaves = [t.detach().cpu().clone().requires_grad_() for t in (x, layer.router, layer.layer_1, layer.layer_2)]
+    x_cpu, router_weight, weight_1, weight_2 = leaves
+    routed = moe_oracle.router(torch.nn.functional.linear(x_cpu, router_weight), k, shared)
+    expected = moe_oracle.looped_moe(x_cpu, routed.scores, routed.top_experts, weight_1, weight_2, experts)
+    objective = (
+        (expected * grad_output.cpu()).sum()
+        + (experts - shared) * coefficient * grad_scale * routed.load_balancing_loss
+        + z_coefficient * grad_scale * routed.z_loss
+    )
+    objective.backward()
+
+    def close(actual, reference, tolerance=1e-4):
+        return (actual.cpu() - reference).abs().max() <= tolerance * reference.abs().max()
+
+    assert close(out.detach(), expected.detach())
+    assert losses[LOAD_BALANCING_LOSS][0].item() == pytest.approx(routed.load_balancing_loss.item(), rel=1e-5)
+    assert losses[ROUTER_Z_LOSS][0].item() == pytest.approx(routed.z_loss.item(), rel=1e-5)
+    assert close(x.grad, x_cpu.grad)
+    assert close(layer.router.grad, router_weight.grad)
+    assert close(layer.layer_1.grad_buffer, weight_1.grad) and close(layer.layer_2.grad_buffer, weight_2.grad)
