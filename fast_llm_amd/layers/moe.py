@@ -129,3 +129,42 @@ class DroplessMoEMLP(torch.nn.Module):
             sparse_map=sparse_map,
         )
         return output.view_as(input_)
+
+    # ---- Hugging Face Mixtral layout ----------------------------------------------------------------------
+    # The reference's Mixtral converter (fast_llm/models/gpt/conversion/mixtral.py:65-82) maps, per block,
+    #   router.weight  <- block_sparse_moe.gate.weight                                   [experts, hidden]
+    #   layer_1.weight <- cat over experts i of (experts.i.w1.weight, experts.i.w3.weight), dim 0
+    #                     (`SplitWeightConverter`, engine/checkpoint/external.py:847-859): [gate_i; up_i] per expert
+    #   layer_2.weight <- cat over i of experts.i.w2.weight along the last dim, transposed
+    #                     (`TransposeSplitWeightConverter`, :862-879): [experts * ffn, hidden]
+    @torch.no_grad()
+    def import_mixtral_weights(self, state_dict: dict[str, torch.Tensor], prefix: str = "") -> None:
+        """Load the weights of one `block_sparse_moe` module of a Hugging Face Mixtral checkpoint (keys
+        `gate.weight`, `experts.{i}.w1|w2|w3.weight` after `prefix`)."""
+        if not self.gated or self.shared_experts != 0:
+            raise ValueError("the Mixtral layout has gated experts and no shared experts")
+
+        def get(name: str) -> torch.Tensor:
+            return state_dict[f"{prefix}{name}"]
+
+        layer_1 = torch.cat(
+            [get(f"experts.{i}.{name}.weight") for i in range(self.experts) for name in ("w1", "w3")], dim=0
+        )
+        layer_2 = torch.cat([get(f"experts.{i}.w2.weight") for i in range(self.experts)], dim=-1).t()
+        for parameter, value in ((self.router, get("gate.weight")), (self.layer_1, layer_1), (self.layer_2, layer_2)):
+            if parameter.shape != value.shape:
+                raise ValueError(f"shape mismatch: {tuple(parameter.shape)} here, {tuple(value.shape)} in the checkpoint")
+            parameter.copy_(value)
+
+    @torch.no_grad()
+    def export_mixtral_weights(self, prefix: str = "") -> dict[str, torch.Tensor]:
+        """The inverse of `import_mixtral_weights`."""
+        if not self.gated or self.shared_experts != 0:
+            raise ValueError("the Mixtral layout has gated experts and no shared experts")
+        out = {f"{prefix}gate.weight": self.router.detach().clone()}
+        for i, (gate_up, down) in enumerate(zip(self.layer_1.chunk(self.experts), self.layer_2.chunk(self.experts))):
+            gate, up = gate_up.chunk(2)
+            out[f"{prefix}experts.{i}.w1.weight"] = gate.clone()
+            out[f"{prefix}experts.{i}.w3.weight"] = up.clone()
+            out[f"{prefix}experts.{i}.w2.weight"] = down.t().contiguous()
+        return out
