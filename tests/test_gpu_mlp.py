@@ -209,3 +209,40 @@ def test_benchmark_configurations_full_size(name, device):
         assert counts.max() > 2.5 * counts.float().mean()
     if workload.empty_experts:
         assert counts[5] == 0 and (actual[4][5 * workload.ffn : 6 * workload.ffn] == 0).all()
+
+
+def test_dynamic_shape_and_micro_batches_accumulate(device):
+    """`dropless_dynamic_shape` (sparse buffers sized by the map instead of the worst case, reference:
+    fast_llm/functional/triton/sparse_copy.py:294-298) gives the same bits as the static shape, and micro-batches of
+    different sizes add up in the gradient buffers (the engine resets `param_grad_is_zero` once per step,
+    fast_llm/engine/multi_stage/fsdp.py:364-372)."""
+    torch.manual_seed(3)
+    layers = {
+        dynamic: DroplessMoEMLP(256, 256, 8, 2, dtype=torch.bfloat16, device=device, dropless_dynamic_shape=dynamic,
+                                full_precision_gradients=True)
+        for dynamic in (False, True)
+    }  # fmt: skip
+    layers[True].load_state_dict(layers[False].state_dict())
+    batches = [torch.randn(tokens, 256, device=device, dtype=torch.bfloat16) for tokens in (300, 517)]
+    results = {}
+    for dynamic, layer in layers.items():
+        outputs, grads = [], []
+        for batch in batches:
+            x = batch.clone().requires_grad_()
+            out = layer(x)
+            out.backward(torch.ones_like(out))
+            outputs.append(out.detach())
+            grads.append(x.grad)
+        results[dynamic] = outputs + grads + [layer.layer_1.grad_buffer.clone(), layer.layer_2.grad_buffer.clone()]
+    for static, dynamic in zip(results[False], results[True]):
+        assert torch.equal(static, dynamic)
+    # Each micro-batch alone, into a fresh buffer: the accumulated buffer is their sum.
+    layer = layers[False]
+    singles = []
+    for batch in batches:
+        layer.layer_1.param_grad_is_zero = layer.layer_2.param_grad_is_zero = True
+        out = layer(batch)
+        out.backward(torch.ones_like(out))
+        singles.append((layer.layer_1.grad_buffer.clone(), layer.layer_2.grad_buffer.clone()))
+    for index in range(2):
+        assert max_rel_err(results[False][4 + index], singles[0][index] + singles[1][index]) <= 1e-6
