@@ -219,3 +219,60 @@ extern "C" int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void
                   row_sparse_dim, static_cast<int>(experts), kInputRowSparse, accumulate, index_dtype, out_dtype, 0, 0, nullptr};
     return run_gemm("fm_input_row_sparse_matmul", args, dtype, stream);
 }
+
+// ---- grouped products with the gated activation fused into the epilogue ------------------------------------
+static int run_fused_gemm(const char *name, GemmArgs args, int dtype, void *stream) {
+    FM_REQUIRE(valid_dtype(dtype) && valid_index_dtype(args.index_dtype), "%s: bad dtype", name);
+    FM_REQUIRE(args.activation >= FM_ACT_GELU && args.activation <= FM_ACT_IDENTITY, "%s: bad activation %d", name,
+               args.activation);
+    FM_REQUIRE(args.rows >= 0 && args.half > 0 && args.inner > 0 && args.num_experts >= 1 &&
+                   args.num_experts < (1 << 20),
+               "%s: bad shape", name);
+    if (args.rows == 0) return FM_OK;
+    FM_REQUIRE(args.lhs && args.rhs, "%s: null tensor", name);
+    if (!mfma_gemm_fusion_eligible(args, dtype))
+        return fail(FM_ERR_UNSUPPORTED,
+                    "%s: needs bf16/fp16, 16-byte aligned K-contiguous operands, K a multiple of 64 and an activation "
+                    "width that is a multiple of 128 (forward) or 8 (backward); run the product and the activation "
+                    "separately",
+                    name);
+    if (int status = mfma_gemm_launch(args, dtype, static_cast<hipStream_t>(stream))) return status;
+    return check_launch(name);
+}
+
+extern "C" int fm_output_sparse_matmul_gated_activation(
+    const void *lhs, const void *rhs, void *layer_1_out, void *activation_out, const void *expert_ends,
+    int64_t row_dim, int64_t activation_dim, int64_t inner_dim, int64_t num_experts, int64_t lhs_stride_row,
+    int64_t lhs_stride_inner, int64_t rhs_stride_inner, int64_t rhs_stride_col, int activation, int dtype,
+    int index_dtype, void *stream) {
+    const char *name = "fm_output_sparse_matmul_gated_activation";
+    FM_REQUIRE(activation_out, "%s: null activation_out", name);
+    GemmArgs args{lhs, rhs, layer_1_out, expert_ends, nullptr, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
+                  rhs_stride_col, 2 * activation_dim, 1, row_dim, 2 * activation_dim, inner_dim, 2 * activation_dim,
+                  static_cast<int>(expert_ends ? num_experts : 1), kOutputSparse, 0, index_dtype, dtype, 0, 0, nullptr};
+    args.fusion = kFusionGatedForward;
+    args.activation = activation;
+    args.fused_out = activation_out;
+    args.fused_stride = activation_dim;
+    args.half = activation_dim;
+    return run_fused_gemm(name, args, dtype, stream);
+}
+
+extern "C" int fm_output_sparse_matmul_gated_activation_backward(
+    const void *lhs, const void *rhs, const void *layer_1_out, void *grad_layer_1_out, void *activation_out,
+    const void *expert_ends, int64_t row_dim, int64_t activation_dim, int64_t inner_dim, int64_t num_experts,
+    int64_t lhs_stride_row, int64_t lhs_stride_inner, int64_t rhs_stride_inner, int64_t rhs_stride_col, int activation,
+    int dtype, int index_dtype, void *stream) {
+    const char *name = "fm_output_sparse_matmul_gated_activation_backward";
+    FM_REQUIRE(layer_1_out && grad_layer_1_out, "%s: null tensor", name);
+    GemmArgs args{lhs, rhs, grad_layer_1_out, expert_ends, nullptr, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
+                  rhs_stride_col, 2 * activation_dim, 1, row_dim, activation_dim, inner_dim, activation_dim,
+                  static_cast<int>(expert_ends ? num_experts : 1), kOutputSparse, 0, index_dtype, dtype, 0, 0, nullptr};
+    args.fusion = kFusionGatedBackward;
+    args.activation = activation;
+    args.fused_in = layer_1_out;
+    args.fused_out = activation_out;
+    args.fused_stride = activation_dim;
+    args.half = activation_dim;
+    return run_fused_gemm(name, args, dtype, stream);
+}

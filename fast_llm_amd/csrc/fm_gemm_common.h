@@ -7,6 +7,15 @@ namespace fm {
 
 enum GemmMode { kOutputSparse = 0, kInputInnerSparse = 1, kInputRowSparse = 2 };
 
+// What the MFMA kernel's epilogue does besides storing the product (output-sparse mode, gated MLP):
+//   kFusionGatedForward: the product is layer 1's output [rows, 2 * half] = [gate | up]; a tile holds 128 gate columns
+//     and the 128 up columns that go with them, `out` (may be null) receives both and `fused_out` [rows, half] receives
+//     act(gate) * up;
+//   kFusionGatedBackward: the product is the gradient of the activation's output [rows, half]; it is not stored:
+//     `fused_in` is layer 1's output, `out` receives the gradient of it (both [rows, 2 * half], same strides) and
+//     `fused_out` (may be null) the recomputed activation output.
+enum GemmFusion { kFusionNone = 0, kFusionGatedForward = 1, kFusionGatedBackward = 2 };
+
 struct GemmArgs {
     const void *lhs;
     const void *rhs;
@@ -25,6 +34,12 @@ struct GemmArgs {
     int out_dtype;
     int tiles_m, tiles_n;
     float *partials;  // workspace of the MFMA kernel for split reductions, or null; set by its launcher
+    int fusion;       // GemmFusion
+    int activation;   // fm_activation tag, for the fused epilogues
+    const void *fused_in;
+    void *fused_out;
+    int64_t fused_stride;  // row stride of fused_out, elements
+    int64_t half;          // columns of the activation output per expert
 };
 
 template <typename OutT>
@@ -43,6 +58,7 @@ __device__ __forceinline__ void store_out_dyn(void *out, int out_dtype, int64_t 
 // Fast path (fm_gemm_mfma.hip). `eligible` says whether the MFMA kernel can take the problem as described by
 // `args` (with `dtype` operands); `launch` fills in the tile counts and launches it.
 bool mfma_gemm_eligible(const GemmArgs &args, int dtype);
+bool mfma_gemm_fusion_eligible(const GemmArgs &args, int dtype);  // with args.fusion set
 int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream);
 
 }  // namespace fm

@@ -30,6 +30,7 @@
 // Results are deterministic: one workgroup per output tile, fixed summation order, no atomics.
 #include <type_traits>
 
+#include "fm_activation_math.h"
 #include "fm_gemm_common.h"
 
 #include <mutex>
@@ -143,8 +144,11 @@ struct TileLoader {
     // `stride`: bytes between rows (K-contiguous) or between K-rows (row-contiguous). Rows >= valid_rows are never
     // stored; a K-contiguous operand gets zeros for them (they lie past the range of the buffer descriptor), a
     // row-contiguous one gets in-range rows in their place.
+    // `split_rows` (K-contiguous only, 0: off): rows 64..127 and 192..255 of the tile are not the rows after 0..63 and
+    // 128..191 but lie `split_rows` rows after them, i.e. tile row n is memory row
+    // (n / 128) * 64 + n % 64 + (n / 64 % 2) * split_rows (the gate and up halves of a gated layer's weight).
     __device__ __forceinline__ void setup(const char *tile_base, int64_t stride, int valid_rows, int num_slices,
-                                          int wave, int lane) {
+                                          int wave, int lane, int split_rows = 0) {
         static_assert(kLoadsPerOperand % 2 == 0, "loads come in (even, odd) pairs");
         fetch_base = tile_base;
         slices_left = num_slices - 1;
@@ -155,7 +159,9 @@ struct TileLoader {
             if constexpr (kContiguousK) {
                 const int row = slot / kChunksPerRow;
                 const int chunk = (slot % kChunksPerRow) ^ k_major_swizzle(row);
-                offset[j] = static_cast<uint32_t>(row * stride + chunk * 16);
+                const int64_t memory_row =
+                    split_rows == 0 ? row : (row >> 7) * 64 + (row & 63) + static_cast<int64_t>((row >> 6) & 1) * split_rows;
+                offset[j] = static_cast<uint32_t>(memory_row * stride + chunk * 16);
             } else {
                 const int k = slot >> 5, position = slot & 31;
                 const int group = (position >> 1) ^ ((k & 3) << 1);
@@ -166,7 +172,8 @@ struct TileLoader {
         }
         // Two loads further on: 128 slots = 16 rows of a K-contiguous slice, 4 K-rows of a row-contiguous one.
         pair_stride = static_cast<uint32_t>((kContiguousK ? 128 / kChunksPerRow : 4) * stride);
-        num_records = kContiguousK ? static_cast<uint32_t>((valid_rows - 1) * stride + kBK * 2) : 0xffffffffu;
+        const int64_t last_row = split_rows == 0 ? valid_rows - 1 : split_rows + kTile / 2 - 1;
+        num_records = kContiguousK ? static_cast<uint32_t>(last_row * stride + kBK * 2) : 0xffffffffu;
         step = kContiguousK ? kBK * 2 : kBK * stride;
     }
 
@@ -264,6 +271,7 @@ __device__ __forceinline__ void mask_tile(FM_LDS(char) * operand_lds, int k0, in
 // ---- which tile ----------------------------------------------------------------------------------------
 struct TileWork {
     int64_t lhs_offset, rhs_offset, out_offset;  // elements
+    int64_t fused_offset;                        // of the tile in `fused_out`, elements
     int rows_valid, cols_valid;
     int64_t k_lo, k_hi;
 };
@@ -312,8 +320,11 @@ __device__ __forceinline__ bool find_row_tile(const GemmArgs &args, int tile, in
 }
 
 __device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int tile_m, int tile_n, TileWork &work) {
-    const int64_t col0 = static_cast<int64_t>(tile_n) * kTile;
-    work.cols_valid = static_cast<int>(min(static_cast<int64_t>(kTile), args.cols - col0));
+    // A tile of the fused gated forward product has 128 gate columns (and their up columns).
+    const bool paired = args.fusion == kFusionGatedForward;
+    const int64_t col0 = static_cast<int64_t>(tile_n) * (paired ? kTile / 2 : kTile);
+    work.cols_valid = paired ? kTile : static_cast<int>(min(static_cast<int64_t>(kTile), args.cols - col0));
+    work.fused_offset = 0;
     work.k_lo = 0;
     work.k_hi = args.inner;
     if (args.mode == kInputRowSparse) {
@@ -337,6 +348,7 @@ __device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int tile_m, i
     if (!find_row_tile(args, tile_m, expert, row0, work.rows_valid)) return false;
     work.lhs_offset = row0 * args.lhs_stride_row;
     work.out_offset = row0 * args.out_stride_row + col0;
+    work.fused_offset = row0 * args.fused_stride + col0;
     if (args.mode == kOutputSparse)
         work.rhs_offset = (static_cast<int64_t>(expert) * args.sparse_size + col0) * args.rhs_stride_col;
     else
@@ -535,6 +547,149 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTiles
     }
 }
 
+// ---- fused epilogues of the gated MLP ---------------------------------------------------------------------
+// Both round the product to T first and compute from the rounded values, exactly what the separate activation
+// kernels would read back from memory, so fused and unfused results are bit-identical.
+
+// The tile is the gradient of the activation output. Per 32-row block: the lane's chunks of layer 1's output (gate and
+// up, 16 bytes each) are requested first, then the accumulators go through LDS as in store_tile, and each staged
+// chunk of 8 gradients becomes 8 gate and 8 up gradients (and, if asked for, the 8 recomputed outputs).
+template <typename T, int kActivation>
+__device__ __forceinline__ void store_tile_gated_backward(const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds,
+                                                          T *grad_layer_1, const T *layer_1, T *activation_out,
+                                                          int64_t stride, int64_t activation_stride, int64_t half,
+                                                          int rows_valid, int cols_valid, int wave, int lane) {
+    constexpr int kChunk = 16 / sizeof(T), kLanesPerRow = kWaveCols / kChunk, kRowsPerRead = 64 / kLanesPerRow;
+    constexpr int kReads = 32 / kRowsPerRead;
+    constexpr int kRowBytes = kWaveCols * sizeof(T) + kEpiloguePadBytes;
+    const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
+    FM_LDS(char) *staging = lds + wave * (32 * kRowBytes);
+    FM_LDS(char) *write_base = staging + (lane & 31) * kRowBytes + (lane >> 5) * 4 * sizeof(T);
+    const int read_row = lane / kLanesPerRow, read_column = (lane % kLanesPerRow) * kChunk;
+    FM_LDS(char) *read_base = staging + read_row * kRowBytes + read_column * sizeof(T);
+    const int column_in_tile = wave_n * kWaveCols + read_column;
+    const bool column_ok = column_in_tile < cols_valid;  // cols_valid is a multiple of 8
+    const int first_row = wave_m * kWaveRows + read_row;
+#pragma unroll
+    for (int i = 0; i < kTilesM; ++i) {
+        const int64_t block_offset = static_cast<int64_t>(first_row + i * 32) * stride + column_in_tile;
+        Vec16<T> gate[kReads], up[kReads];
+        bool valid[kReads];
+#pragma unroll
+        for (int t = 0; t < kReads; ++t) {
+            valid[t] = first_row + i * 32 + t * kRowsPerRead < rows_valid && column_ok;
+            if (valid[t]) {
+                const T *source = layer_1 + block_offset + static_cast<int64_t>(t) * kRowsPerRead * stride;
+                gate[t] = load16_stream(source);
+                up[t] = load16_stream(source + half);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kTilesN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                Vec16x4<T> group;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) group.v[c] = from_float<T>(acc[i][j][4 * g + c]);
+                *reinterpret_cast<FM_LDS(u32x2_t) *>(write_base + (j * 32 + 8 * g) * sizeof(T)) =
+                    __builtin_bit_cast(u32x2_t, group);
+            }
+        asm volatile("" ::: "memory");  // one wavefront, in-order LDS: no barrier needed (see store_tile)
+        u32x4_t staged[kReads];
+#pragma unroll
+        for (int t = 0; t < kReads; ++t)
+            staged[t] = *reinterpret_cast<FM_LDS(u32x4_t) *>(read_base + t * kRowsPerRead * kRowBytes);
+#pragma unroll
+        for (int t = 0; t < kReads; ++t) {
+            if (!valid[t]) continue;
+            const Vec16<T> grad = __builtin_bit_cast(Vec16<T>, staged[t]);
+            Vec16<T> grad_gate, grad_up, recomputed;
+#pragma unroll
+            for (int c = 0; c < kChunk; ++c) {
+                float out;
+                const float derivative = activation_backward<kActivation>(to_float(gate[t].v[c]), out);
+                const float g = to_float(grad.v[c]), other = to_float(up[t].v[c]);
+                grad_gate.v[c] = from_float<T>(derivative * other * g);
+                grad_up.v[c] = from_float<T>(out * g);
+                recomputed.v[c] = from_float<T>(out * other);
+            }
+            const int64_t row_offset = static_cast<int64_t>(t) * kRowsPerRead;
+            T *target = grad_layer_1 + block_offset + row_offset * stride;
+            store16_stream(target, grad_gate);
+            store16_stream(target + half, grad_up);
+            if (activation_out != nullptr)
+                store16_stream(activation_out + static_cast<int64_t>(first_row + i * 32 + row_offset) * activation_stride +
+                                   column_in_tile,
+                               recomputed);
+        }
+        asm volatile("" ::: "memory");
+    }
+}
+
+// The tile is 128 gate columns and their 128 up columns of layer 1's output; a wavefront holds gate columns in its
+// accumulators j = 0, 1 and the matching up columns in j = 2, 3. Per 32-row block it stages, per row, 64 gate values,
+// 64 up values and 64 outputs act(gate) * up, and stores each as 128-byte row segments.
+template <typename T, int kActivation>
+__device__ __forceinline__ void store_tile_gated_forward(const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds,
+                                                         T *layer_1, T *activation_out, int64_t stride,
+                                                         int64_t activation_stride, int64_t half, int rows_valid,
+                                                         int wave, int lane) {
+    static_assert(kTilesN == 4 && kWaveCols == 128, "two gate and two up accumulators per row block");
+    constexpr int kChunk = 16 / sizeof(T);                 // 8
+    constexpr int kSegment = kWaveCols / 2;                // 64 columns per segment
+    constexpr int kChunksPerRow = 3 * kSegment / kChunk;   // 24
+    constexpr int kReads = 32 * kChunksPerRow / 64;        // 12
+    constexpr int kRowBytes = 3 * kSegment * sizeof(T) + kEpiloguePadBytes;
+    const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
+    FM_LDS(char) *staging = lds + wave * (32 * kRowBytes);
+    FM_LDS(char) *write_base = staging + (lane & 31) * kRowBytes + (lane >> 5) * 4 * sizeof(T);
+#pragma unroll
+    for (int i = 0; i < kTilesM; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                Vec16x4<T> gate, up, result;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    gate.v[c] = from_float<T>(acc[i][j][4 * g + c]);
+                    up.v[c] = from_float<T>(acc[i][j + 2][4 * g + c]);
+                    result.v[c] =
+                        from_float<T>(activation_forward<kActivation>(to_float(gate.v[c])) * to_float(up.v[c]));
+                }
+                FM_LDS(char) *position = write_base + (j * 32 + 8 * g) * sizeof(T);
+                *reinterpret_cast<FM_LDS(u32x2_t) *>(position) = __builtin_bit_cast(u32x2_t, gate);
+                *reinterpret_cast<FM_LDS(u32x2_t) *>(position + kSegment * sizeof(T)) = __builtin_bit_cast(u32x2_t, up);
+                *reinterpret_cast<FM_LDS(u32x2_t) *>(position + 2 * kSegment * sizeof(T)) =
+                    __builtin_bit_cast(u32x2_t, result);
+            }
+        asm volatile("" ::: "memory");
+        u32x4_t staged[kReads];
+#pragma unroll
+        for (int t = 0; t < kReads; ++t) {
+            const int id = t * 64 + lane;
+            staged[t] = *reinterpret_cast<FM_LDS(u32x4_t) *>(staging + (id / kChunksPerRow) * kRowBytes +
+                                                             (id % kChunksPerRow) * 16);
+        }
+#pragma unroll
+        for (int t = 0; t < kReads; ++t) {
+            const int id = t * 64 + lane;
+            const int row = wave_m * kWaveRows + i * 32 + id / kChunksPerRow, chunk = id % kChunksPerRow;
+            const int segment = chunk / (kSegment / kChunk);
+            const int column = wave_n * kSegment + (chunk % (kSegment / kChunk)) * kChunk;
+            if (row >= rows_valid) continue;
+            if (segment == 2) {
+                __builtin_nontemporal_store(
+                    staged[t], reinterpret_cast<u32x4_t *>(activation_out + row * activation_stride + column));
+            } else if (layer_1 != nullptr) {
+                __builtin_nontemporal_store(
+                    staged[t], reinterpret_cast<u32x4_t *>(layer_1 + row * stride + segment * half + column));
+            }
+        }
+        asm volatile("" ::: "memory");
+    }
+}
+
 __device__ __forceinline__ void store_result(const GemmArgs &args, const TileWork &work,
                                              const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds, int wave,
                                              int lane) {
@@ -575,8 +730,10 @@ __device__ __forceinline__ void store_partial(const f32x16_t (&acc)[kTilesM][kTi
 }
 
 // kMasked: the row-sparse product, whose reduction range [k_lo, k_hi) is ragged.
-template <typename T, bool kLhsContiguousK, bool kRhsContiguousK, bool kMasked>
+// kFusion: a GemmFusion, the epilogue to run instead of the plain store.
+template <typename T, bool kLhsContiguousK, bool kRhsContiguousK, bool kMasked, int kFusion = kFusionNone>
 __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_kernel(GemmArgs args) {
+    static_assert(kFusion == kFusionNone || (kRhsContiguousK && !kMasked), "fused epilogues: output-sparse, K-major rhs");
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);  // C-style: address-space cast
 
@@ -613,7 +770,8 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         load_lhs.setup(uniform_pointer(lhs), (kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner) * sizeof(T),
                        work.rows_valid, num_slices, wave, lane);
         load_rhs.setup(uniform_pointer(rhs), (kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner) * sizeof(T),
-                       work.cols_valid, num_slices, wave, lane);
+                       work.cols_valid, num_slices, wave, lane,
+                       kFusion == kFusionGatedForward ? static_cast<int>(args.half) : 0);
     }
 
     f32x16_t acc[kTilesM][kTilesN];
@@ -759,8 +917,25 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
 
     if (piece_slot < 0 && args.accumulate != 0 && num_slices == 0) return;  // nothing to add
     __syncthreads();  // all wavefronts are done reading operand slices; LDS becomes the staging area
-    if (piece_slot >= 0) store_partial(acc, args.partials + static_cast<int64_t>(piece_slot) * kPartialFloats, wave, lane);
-    else store_result(args, work, acc, lds, wave, lane);
+    if constexpr (kFusion == kFusionGatedForward) {
+        T *layer_1 = args.out == nullptr ? nullptr : static_cast<T *>(args.out) + work.out_offset;
+        FM_DISPATCH_ACTIVATION(args.activation, kActivation,
+                               store_tile_gated_forward<T, kActivation>(
+                                   acc, lds, layer_1, static_cast<T *>(args.fused_out) + work.fused_offset,
+                                   args.out_stride_row, args.fused_stride, args.half, work.rows_valid, wave, lane));
+    } else if constexpr (kFusion == kFusionGatedBackward) {
+        T *recomputed = args.fused_out == nullptr ? nullptr : static_cast<T *>(args.fused_out) + work.fused_offset;
+        FM_DISPATCH_ACTIVATION(args.activation, kActivation,
+                               store_tile_gated_backward<T, kActivation>(
+                                   acc, lds, static_cast<T *>(args.out) + work.out_offset,
+                                   static_cast<const T *>(args.fused_in) + work.out_offset, recomputed,
+                                   args.out_stride_row, args.fused_stride, args.half, work.rows_valid, work.cols_valid,
+                                   wave, lane));
+    } else {
+        if (piece_slot >= 0)
+            store_partial(acc, args.partials + static_cast<int64_t>(piece_slot) * kPartialFloats, wave, lane);
+        else store_result(args, work, acc, lds, wave, lane);
+    }
 }
 
 // Adds the pieces of each tile whose reduction the main kernel split, in piece order, and stores the sums.
@@ -810,9 +985,9 @@ static int allow_big_lds(const void *kernel) {
     return FM_OK;
 }
 
-template <typename T, bool kLhsK, bool kRhsK, bool kMasked>
+template <typename T, bool kLhsK, bool kRhsK, bool kMasked, int kFusion = kFusionNone>
 static int launch_instance(const GemmArgs &args, hipStream_t stream) {
-    auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK, kMasked>;
+    auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK, kMasked, kFusion>;
     static bool configured = false;  // setting the attribute twice from racing threads is harmless
     if (!configured) {
         if (int status = allow_big_lds(reinterpret_cast<const void *>(kernel))) return status;
@@ -837,6 +1012,8 @@ static int launch_instance(const GemmArgs &args, hipStream_t stream) {
 template <typename T>
 static int launch_layout(const GemmArgs &args, hipStream_t stream) {
     const bool lhs_k = args.lhs_stride_inner == 1, rhs_k = args.rhs_stride_inner == 1;
+    if (args.fusion == kFusionGatedForward) return launch_instance<T, true, true, false, kFusionGatedForward>(args, stream);
+    if (args.fusion == kFusionGatedBackward) return launch_instance<T, true, true, false, kFusionGatedBackward>(args, stream);
     // Only the row-sparse product with a map has a ragged reduction range.
     const bool masked = args.mode == kInputRowSparse && args.expert_ends != nullptr;
 #define FM_LAUNCH(LHS, RHS) \
@@ -917,6 +1094,21 @@ float *split_workspace(hipStream_t stream) {
 }
 }  // namespace
 
+// The fused epilogues exist for one layout: both operands K-contiguous, output-sparse mode, T in and out, whole
+// column tiles (the activation width a multiple of 128 for the forward, of 8 for the backward).
+bool mfma_gemm_fusion_eligible(const GemmArgs &args, int dtype) {
+    if (!mfma_gemm_eligible(args, dtype) || args.mode != kOutputSparse || args.out_dtype != dtype || args.accumulate)
+        return false;
+    if (args.lhs_stride_inner != 1 || args.rhs_stride_inner != 1) return false;
+    if (!aligned16(args.fused_out) || !aligned16(args.fused_in) || args.fused_stride % 8 != 0 || args.half % 8 != 0)
+        return false;
+    if (args.fusion == kFusionGatedForward) {
+        // The up rows of a tile are addressed with 32-bit byte offsets from its gate rows.
+        if (args.half % (kTile / 2) != 0 || (args.half + kTile) * args.rhs_stride_col * 2 >= (int64_t(1) << 32)) return false;
+    }
+    return true;
+}
+
 int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream) {
     if (args.mode == kInputRowSparse) {
         args.tiles_m = static_cast<int>((args.sparse_size + kTile - 1) / kTile) * args.num_experts;
@@ -925,12 +1117,13 @@ int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream) {
         args.tiles_m = static_cast<int>((args.rows + kTile - 1) / kTile + (args.expert_ends ? args.num_experts : 0));
     }
     args.tiles_n = static_cast<int>((args.cols + kTile - 1) / kTile);
+    if (args.fusion == kFusionGatedForward) args.tiles_n = static_cast<int>(args.half / (kTile / 2));
     if (static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31) - 1024)
         return fail(FM_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
     // Splitting the last round's reductions can pay when the rounds are few and the reduction is long.
     args.partials = nullptr;
     constexpr int kMaxRoundsToSplit = 16;
-    if (args.mode != kInputRowSparse && args.inner / kBK >= 2 * kMinPieceSlices &&
+    if (args.fusion == kFusionNone && args.mode != kInputRowSparse && args.inner / kBK >= 2 * kMinPieceSlices &&
         static_cast<int64_t>(args.tiles_m) * args.tiles_n <= kMaxRoundsToSplit * kRound && split_enabled())
         args.partials = split_workspace(stream);
     return dtype == FM_DTYPE_BF16 ? launch_layout<bf16_t>(args, stream) : launch_layout<f16_t>(args, stream);

@@ -103,6 +103,84 @@ def torch_mlp_activation(input_: torch.Tensor, gated: bool, activation_type: Act
     return activation_type.activation_fn(input_)
 
 
+def _fusable(lhs: torch.Tensor, weight_t: torch.Tensor, gated: bool, sparse_map: SparseMap | None, *biases) -> bool:
+    """Whether a layer-1 product / layer-2 input gradient may take the kernel with the gated activation in its
+    epilogue; the library has the last word (`NotImplementedError`: shapes it cannot tile)."""
+    return (
+        gated
+        and sparse_map is not None
+        and all(bias is None for bias in biases)
+        and lhs.dtype in (torch.bfloat16, torch.float16)
+        and weight_t.dtype == lhs.dtype
+        and lhs.dim() == 2
+        and lhs.stride(1) == 1
+        and weight_t.stride(0) == 1
+    )
+
+
+def _launch_fused(name: str, lhs: torch.Tensor, weight_t: torch.Tensor, tensors: tuple, sparse_map: SparseMap,
+                  activation_dim: int, activation_type: ActivationType, label_columns: int) -> None:  # fmt: skip
+    device = _lib.require_device(lhs, weight_t, *tensors)
+    _lib.call(
+        name,
+        device,
+        _lib.ptr(lhs.detach()),
+        _lib.ptr(weight_t.detach()),
+        *(_lib.ptr(tensor) for tensor in tensors),
+        _lib.ptr(sparse_map.expert_ends),
+        lhs.size(0),
+        activation_dim,
+        lhs.size(1),
+        sparse_map.num_experts,
+        lhs.stride(0),
+        lhs.stride(1),
+        weight_t.stride(0),
+        weight_t.stride(1),
+        _activation_tag(activation_type),
+        _lib.dtype_tag(lhs.dtype),
+        _lib.index_tag(sparse_map.expert_ends.dtype),
+        label=f"{name}[{lhs.size(0)}x{label_columns}x{lhs.size(1)}]",
+    )
+
+
+def gated_layer_1_forward(
+    input_: torch.Tensor, weight_1: torch.Tensor, sparse_map: SparseMap, activation_type: ActivationType, keep_layer_1: bool
+) -> tuple[torch.Tensor | None, torch.Tensor]:
+    """
+    (layer-1 output or None, activation output) of a gated sparse MLP in one kernel: `output_sparse_matmul` with
+    `triton_mlp_activation_forward` in its epilogue (reference: the two calls at fast_llm/functional/triton/mlp.py:246-258).
+    Bit-identical to the two separate kernels. Raises NotImplementedError for shapes the fused kernel does not take.
+    """
+    activation_dim = weight_1.size(0) // sparse_map.num_experts // 2
+    layer_1 = input_.new_empty(input_.size(0), 2 * activation_dim) if keep_layer_1 else None
+    output = input_.new_empty(input_.size(0), activation_dim)
+    _launch_fused(
+        "fm_output_sparse_matmul_gated_activation", input_, weight_1.t(), (layer_1, output), sparse_map,
+        activation_dim, activation_type, 2 * activation_dim,
+    )  # fmt: skip
+    return layer_1, output
+
+
+def gated_layer_2_input_backward(
+    grad_output: torch.Tensor, weight_2_t: torch.Tensor, sparse_map: SparseMap, layer_1: torch.Tensor,
+    activation_type: ActivationType, recompute: bool,
+) -> tuple[torch.Tensor, torch.Tensor | None]:  # fmt: skip
+    """
+    (gradient of the layer-1 output, recomputed activation output or None): the layer-2 input gradient
+    `output_sparse_matmul(grad_output, weight_2_t)` handed tile by tile to `triton_mlp_activation_backward` instead
+    of being stored (reference: fast_llm/functional/triton/mlp.py:352-359, 373-375). Bit-identical to the two kernels.
+    """
+    assert layer_1.is_contiguous()
+    activation_dim = layer_1.size(1) // 2
+    grad_layer_1 = torch.empty_like(layer_1)
+    output = layer_1.new_empty(layer_1.size(0), activation_dim) if recompute else None
+    _launch_fused(
+        "fm_output_sparse_matmul_gated_activation_backward", grad_output, weight_2_t,
+        (layer_1.detach(), grad_layer_1, output), sparse_map, activation_dim, activation_type, activation_dim,
+    )  # fmt: skip
+    return grad_layer_1, output
+
+
 def mlp_forward(
     input_: torch.Tensor,
     scores: torch.Tensor | None,
@@ -133,18 +211,25 @@ def mlp_forward(
     input_shape = input_.shape
     intermediate_0 = input_ if sparse_map is None else copy_dense_to_sparse_forward(input_, sparse_map)[0]
 
-    # Layer 1
-    intermediate_1, _ = output_parallel_linear_forward(
-        intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
-    )
+    # Layer 1 and activation: one kernel where the library has one, else the reference's two steps.
+    intermediate_2 = None
+    if KernelConfig.fuse_activation and _fusable(intermediate_0, weight_1.t(), gated, sparse_map, bias_1):
+        try:
+            intermediate_1, intermediate_2 = gated_layer_1_forward(
+                intermediate_0, weight_1, sparse_map, activation_type, training and not recompute_level.recompute_layer_1
+            )
+        except NotImplementedError:
+            pass
+    if intermediate_2 is None:
+        intermediate_1, _ = output_parallel_linear_forward(
+            intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
+        )
+        intermediate_2, _ = mlp_activation_forward(intermediate_1, gated, activation_type)
 
     if recompute_level.recompute_sparse_input:
         intermediate_0 = None
     else:
         input_ = None
-
-    # Activation
-    intermediate_2, _ = mlp_activation_forward(intermediate_1, gated, activation_type)
     if recompute_level.recompute_layer_1:
         intermediate_1 = None
 
@@ -224,13 +309,6 @@ def mlp_backward(grad_output: torch.Tensor, context: list[typing.Any]) -> tuple[
     else:
         grad_output, grad_scores = copy_sparse_to_dense_backward(grad_output, (sparse_map, intermediate_3, scores))
 
-    # Layer 2 input grad
-    weight_2_t = maybe_transpose(weight_2, transposed_layer_2_weight)
-    if sparse_map is None:
-        grad_intermediate_2 = grad_output.matmul(weight_2_t)
-    else:
-        grad_intermediate_2 = output_sparse_matmul(grad_output, weight_2_t, sparse_map)
-
     # Sparse input recomputation
     if intermediate_0 is None:
         intermediate_0 = input_ if sparse_map is None else copy_dense_to_sparse_forward(input_, sparse_map)[0]
@@ -241,13 +319,29 @@ def mlp_backward(grad_output: torch.Tensor, context: list[typing.Any]) -> tuple[
             intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
         )[0]
 
-    # Activation recomputation and/or backward
-    grad_intermediate_1, intermediate_2_ = mlp_activation_backward(
-        grad_intermediate_2.contiguous(), (intermediate_1, gated, activation_type), intermediate_2 is None
-    )
+    # Layer 2 input grad, then activation recomputation and/or backward: in one kernel where the library has one
+    # (the reference computes the layer 2 input grad before the two recomputations; they are independent).
+    weight_2_t = maybe_transpose(weight_2, transposed_layer_2_weight)
+    grad_intermediate_1 = None
+    if KernelConfig.fuse_activation and _fusable(grad_output, weight_2_t, gated, sparse_map):
+        try:
+            grad_intermediate_1, intermediate_2_ = gated_layer_2_input_backward(
+                grad_output, weight_2_t, sparse_map, intermediate_1, activation_type, intermediate_2 is None
+            )
+        except NotImplementedError:
+            pass
+    if grad_intermediate_1 is None:
+        if sparse_map is None:
+            grad_intermediate_2 = grad_output.matmul(weight_2_t)
+        else:
+            grad_intermediate_2 = output_sparse_matmul(grad_output, weight_2_t, sparse_map)
+        grad_intermediate_1, intermediate_2_ = mlp_activation_backward(
+            grad_intermediate_2.contiguous(), (intermediate_1, gated, activation_type), intermediate_2 is None
+        )
+        del grad_intermediate_2
 
     # Layer 2 parameter grad
-    del grad_intermediate_2, intermediate_1
+    del intermediate_1
     update_linear_gradients(
         intermediate_2_ if intermediate_2 is None else intermediate_2,
         weight_2,

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 3
+#define FM_VERSION 4
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -231,6 +231,36 @@ int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void *out, cons
                                int64_t lhs_stride_inner, int64_t rhs_stride_inner, int64_t rhs_stride_col,
                                int64_t out_stride_row, int64_t out_stride_col, int accumulate, int dtype,
                                int out_dtype, int index_dtype, void *stream);
+
+/* Layer 1 of a gated MLP with the activation fused into the product's epilogue: what the reference does with
+ * `output_sparse_matmul` (fast_llm/functional/triton/sparse_linear.py:261-306) followed by
+ * `triton_mlp_activation_forward` (fast_llm/functional/triton/mlp.py:29-67, 131-154), as called from `mlp_forward`
+ * (:246-258). lhs [row_dim, inner_dim]; rhs [inner_dim, num_experts * 2 * activation_dim] (per expert the gate
+ * columns, then the up columns); layer_1_out [row_dim, 2 * activation_dim] contiguous, or null when it is not kept;
+ * activation_out [row_dim, activation_dim] contiguous = act(gate) * up, computed from the rounded product, so both
+ * outputs are bit-identical to the two separate calls. Returns FM_ERR_UNSUPPORTED when the shape does not fit the
+ * matrix-core kernel (fp32; operands not contiguous along inner_dim; inner_dim not a multiple of 64; activation_dim
+ * not a multiple of 128): call the product and the activation separately then. */
+int fm_output_sparse_matmul_gated_activation(const void *lhs, const void *rhs, void *layer_1_out, void *activation_out,
+                                             const void *expert_ends, int64_t row_dim, int64_t activation_dim,
+                                             int64_t inner_dim, int64_t num_experts, int64_t lhs_stride_row,
+                                             int64_t lhs_stride_inner, int64_t rhs_stride_inner, int64_t rhs_stride_col,
+                                             int activation, int dtype, int index_dtype, void *stream);
+
+/* The gradient of layer 1's output in the backward of a gated MLP: the product of the reference's layer-2 input
+ * gradient `output_sparse_matmul(grad_output, weight_2_t, sparse_map)` (fast_llm/functional/triton/mlp.py:352-359)
+ * is not stored but handed, tile by tile, to the activation backward `triton_mlp_activation_backward` (:70-128,
+ * 157-185, called at :373-375). lhs [row_dim, inner_dim]; rhs [inner_dim, num_experts * activation_dim];
+ * layer_1_out and grad_layer_1_out [row_dim, 2 * activation_dim] contiguous; activation_out
+ * [row_dim, activation_dim] or null: the recomputed activation output. Bit-identical to the two separate calls.
+ * FM_ERR_UNSUPPORTED as above (activation_dim a multiple of 8 is enough here). */
+int fm_output_sparse_matmul_gated_activation_backward(const void *lhs, const void *rhs, const void *layer_1_out,
+                                                      void *grad_layer_1_out, void *activation_out,
+                                                      const void *expert_ends, int64_t row_dim, int64_t activation_dim,
+                                                      int64_t inner_dim, int64_t num_experts, int64_t lhs_stride_row,
+                                                      int64_t lhs_stride_inner, int64_t rhs_stride_inner,
+                                                      int64_t rhs_stride_col, int activation, int dtype,
+                                                      int index_dtype, void *stream);
 
 #ifdef __cplusplus
 }

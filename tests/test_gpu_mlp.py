@@ -15,7 +15,10 @@ from tests.helpers import REFERENCE_FIXTURES, max_rel_err, rms_diff
 pytestmark = pytest.mark.gpu
 
 
-def _run_dropless(inputs, workload, device, recompute_level=MLPRecomputeLevel.none, grad_dtype=None, repeat=1):
+def _run_dropless(
+    inputs, workload, device, recompute_level=MLPRecomputeLevel.none, grad_dtype=None, repeat=1,
+    activation=ActivationType.silu,
+):  # fmt: skip
     x = inputs.hidden_states.to(device).requires_grad_(True)
     scores = inputs.scores.to(device).requires_grad_(True)
     weight_1 = inputs.weight_1.to(device).requires_grad_(True)
@@ -25,7 +28,7 @@ def _run_dropless(inputs, workload, device, recompute_level=MLPRecomputeLevel.no
     sparse_map = get_sparse_map(inputs.top_experts.to(device), workload.experts)
     for _ in range(repeat):
         output = mlp_autograd(
-            x, scores, weight_1, None, weight_2, None, True, ActivationType.silu, None, False, True,
+            x, scores, weight_1, None, weight_2, None, True, activation, None, False, True,
             recompute_level, True, sparse_map,
         )
         output.backward(inputs.grad_output.to(device))
@@ -246,3 +249,27 @@ def test_dynamic_shape_and_micro_batches_accumulate(device):
         singles.append((layer.layer_1.grad_buffer.clone(), layer.layer_2.grad_buffer.clone()))
     for index in range(2):
         assert max_rel_err(results[False][4 + index], singles[0][index] + singles[1][index]) <= 1e-6
+
+
+@pytest.mark.parametrize("recompute_level", list(MLPRecomputeLevel))
+@pytest.mark.parametrize("activation", ["silu", "gelu", "relu", "squared_relu", "identity"])
+def test_fused_activation_epilogues_are_bit_identical(activation, recompute_level, device, monkeypatch):
+    """The gated activation inside the grouped products' epilogues (forward in layer 1, backward in the layer 2
+    input gradient) against the separate kernels: every output and gradient, bit for bit, ragged experts included."""
+    from fast_llm_amd import _lib
+    from fast_llm_amd.functional.config import KernelConfig
+
+    workload = MoEWorkload("fused", 700, 192, 384, 5, 2, torch.bfloat16)
+    inputs = make_inputs(workload, seed=9)
+    results = {}
+    for fused in (True, False):
+        monkeypatch.setattr(KernelConfig, "fuse_activation", fused)
+        with _lib.KernelTimer() as timer:
+            results[fused] = _run_dropless(
+                inputs, workload, device, recompute_level=recompute_level, activation=ActivationType(activation)
+            )
+        labels = set(timer.durations_ms())
+        assert any("gated_activation" in label for label in labels) == fused
+        assert any(label.startswith("fm_mlp_activation") for label in labels) == (not fused)
+    for fused, separate in zip(results[True], results[False]):
+        assert torch.equal(fused, separate)
