@@ -483,9 +483,10 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int
 // what `out` holds: then they stay fp32 and are rounded once after the addition), a group goes to LDS as one 8- or
 // 16-byte write, and the staged rows are read back as 16-byte chunks in row-major order, all reads of a 32-row block
 // before the first store, so that a store instruction covers full 256-byte row segments.
-template <typename OutT, bool kAccumulate>
-__device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds, OutT *out,
-                                           int64_t stride, int rows_valid, int cols_valid, int wave, int lane) {
+// `source(i)` yields the wavefront's accumulators of its i-th block of 32 rows, as something indexed [j][register].
+template <typename OutT, bool kAccumulate, typename Source>
+__device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, OutT *out, int64_t stride,
+                                           int rows_valid, int cols_valid, int wave, int lane) {
     using StageT = std::conditional_t<kAccumulate, float, OutT>;
     constexpr int kChunk = 16 / sizeof(StageT);         // elements per 16-byte chunk
     constexpr int kLanesPerRow = kWaveCols / kChunk;    // 16 or 32
@@ -504,13 +505,14 @@ __device__ __forceinline__ void store_tile(const f32x16_t (&acc)[kTilesM][kTiles
     OutT *pointer = out + first_row * stride + column_in_tile;
 #pragma unroll
     for (int i = 0; i < kTilesM; ++i) {
+        auto &&block = source(i);
 #pragma unroll
         for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 Vec16x4<StageT> group;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) group.v[c] = from_float<StageT>(acc[i][j][4 * g + c]);
+                for (int c = 0; c < 4; ++c) group.v[c] = from_float<StageT>(block[j][4 * g + c]);
                 using Raw = std::conditional_t<sizeof(StageT) == 4, u32x4_t, u32x2_t>;
                 *reinterpret_cast<FM_LDS(Raw) *>(write_base + (j * 32 + 8 * g) * sizeof(StageT)) =
                     __builtin_bit_cast(Raw, group);
@@ -690,17 +692,19 @@ __device__ __forceinline__ void store_tile_gated_forward(const f32x16_t (&acc)[k
     }
 }
 
-__device__ __forceinline__ void store_result(const GemmArgs &args, const TileWork &work,
-                                             const f32x16_t (&acc)[kTilesM][kTilesN], FM_LDS(char) * lds, int wave,
-                                             int lane) {
+template <typename Source>
+__device__ __forceinline__ void store_result(const GemmArgs &args, const TileWork &work, Source &&source,
+                                             FM_LDS(char) * lds, int wave, int lane) {
     const bool accumulate = args.accumulate != 0;
     auto store = [&](auto *out) {
         if (accumulate)
-            store_tile<std::remove_pointer_t<decltype(out)>, true>(acc, lds, out + work.out_offset, args.out_stride_row,
-                                                                   work.rows_valid, work.cols_valid, wave, lane);
+            store_tile<std::remove_pointer_t<decltype(out)>, true>(source, lds, out + work.out_offset,
+                                                                   args.out_stride_row, work.rows_valid,
+                                                                   work.cols_valid, wave, lane);
         else
-            store_tile<std::remove_pointer_t<decltype(out)>, false>(acc, lds, out + work.out_offset, args.out_stride_row,
-                                                                    work.rows_valid, work.cols_valid, wave, lane);
+            store_tile<std::remove_pointer_t<decltype(out)>, false>(source, lds, out + work.out_offset,
+                                                                    args.out_stride_row, work.rows_valid,
+                                                                    work.cols_valid, wave, lane);
     };
     if (args.out_dtype == FM_DTYPE_F32) store(static_cast<float *>(args.out));
     else if (args.out_dtype == FM_DTYPE_BF16) store(static_cast<bf16_t *>(args.out));
@@ -934,48 +938,56 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     } else {
         if (piece_slot >= 0)
             store_partial(acc, args.partials + static_cast<int64_t>(piece_slot) * kPartialFloats, wave, lane);
-        else store_result(args, work, acc, lds, wave, lane);
+        else
+            store_result(
+                args, work, [&](int i) -> const f32x16_t(&)[kTilesN] { return acc[i]; }, lds, wave, lane);
     }
 }
 
 // Adds the pieces of each tile whose reduction the main kernel split, in piece order, and stores the sums.
-// One workgroup per tile of the last round.
-__global__ __launch_bounds__(kMfmaThreads) void grouped_gemm_reduce_kernel(GemmArgs args) {
+// One single-wavefront workgroup per quarter of a tile (what one wavefront of the main kernel computed), so that the
+// few tiles of a last round still spread over all CUs.
+constexpr int kReduceLdsBytes = kWaves * 32 * (kWaveCols * 4 + kEpiloguePadBytes);  // the staging areas of store_tile
+__global__ __launch_bounds__(64) void grouped_gemm_reduce_kernel(GemmArgs args) {
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);
     const SplitPlan plan = plan_split(args);
-    const int index = blockIdx.x;
+    const int index = blockIdx.x / kWaves;
     if (plan.pieces == 1 || index >= plan.tail) return;
     int tile_m, tile_n;
     TileWork work;
     tile_coordinates(plan.whole + index, plan.tiles_m, args.tiles_n, tile_m, tile_n);
     if (!resolve_tile(args, tile_m, tile_n, work)) return;
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    f32x16_t acc[kTilesM][kTilesN];
-#pragma unroll
-    for (int i = 0; i < kTilesM; ++i)
+    const int lane = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x % kWaves));
+    // One block of 32 rows at a time: 64 registers of sums, the loads of a piece all in flight together.
+    struct RowBlock {
+        f32x16_t values[kTilesN];
+        __device__ const f32x16_t &operator[](int j) const { return values[j]; }
+    };
+    auto summed_block = [&](int i) {
+        RowBlock block;
 #pragma unroll
         for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    for (int piece = 0; piece < plan.pieces; ++piece) {
-        const float *partial = partial_of_lane(
-            args.partials + static_cast<int64_t>(piece * plan.tail + index) * kPartialFloats, wave, lane);
-#pragma unroll
-        for (int i = 0; i < kTilesM; ++i)
+            for (int v = 0; v < 16; ++v) block.values[j][v] = 0.f;
+        for (int piece = 0; piece < plan.pieces; ++piece) {
+            const float *partial =
+                partial_of_lane(args.partials + static_cast<int64_t>(piece * plan.tail + index) * kPartialFloats, wave,
+                                lane) +
+                i * kTilesN * 4 * 256;
 #pragma unroll
             for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const f32x4_t value =
-                        *reinterpret_cast<const f32x4_t *>(partial + ((i * kTilesN + j) * 4 + g) * 256);
+                    const f32x4_t value = *reinterpret_cast<const f32x4_t *>(partial + (j * 4 + g) * 256);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c)
-                        acc[i][j][4 * g + c] += value[c];
+                    for (int c = 0; c < 4; ++c) block.values[j][4 * g + c] += value[c];
                 }
-    }
-    store_result(args, work, acc, lds, wave, lane);
+        }
+        return block;
+    };
+    store_result(args, work, summed_block, lds, wave, lane);
 }
 
 // ---- host side -----------------------------------------------------------------------------------------
@@ -1001,10 +1013,12 @@ static int launch_instance(const GemmArgs &args, hipStream_t stream) {
     if (args.partials != nullptr) {
         static bool reduce_configured = false;
         if (!reduce_configured) {
-            if (int status = allow_big_lds(reinterpret_cast<const void *>(grouped_gemm_reduce_kernel))) return status;
+            hipError_t error = hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_reduce_kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kReduceLdsBytes);
+            if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
             reduce_configured = true;
         }
-        grouped_gemm_reduce_kernel<<<kRound, kMfmaThreads, kLdsBytes, stream>>>(args);
+        grouped_gemm_reduce_kernel<<<kRound * kWaves, 64, kReduceLdsBytes, stream>>>(args);
     }
     return FM_OK;
 }
