@@ -273,3 +273,55 @@ def test_fused_activation_epilogues_are_bit_identical(activation, recompute_leve
         assert any(label.startswith("fm_mlp_activation") for label in labels) == (not fused)
     for fused, separate in zip(results[True], results[False]):
         assert torch.equal(fused, separate)
+
+
+def test_step_replays_from_a_hip_graph(device):
+    """Forward + backward of the block (sparse map included) captured once in a HIP graph and replayed with new
+    inputs: every replay, with eager work and synchronisations in between, equals the eager result bit for bit.
+    The warm-up runs on the capture stream, which also gives that stream its split-reduction workspace (the library
+    does not allocate while a stream is being captured)."""
+    torch.manual_seed(5)
+    tokens, hidden, ffn, experts, k = 512, 256, 2048, 4, 2  # few tiles, long reduction: the split path is taken
+    layer = DroplessMoEMLP(hidden, ffn, experts, k, dtype=torch.bfloat16, device=device)
+    inputs = [torch.randn(tokens, hidden, device=device, dtype=torch.bfloat16) for _ in range(3)]
+    grad_output = torch.randn(tokens, hidden, device=device, dtype=torch.bfloat16)
+
+    def eager(x):
+        x = x.clone().requires_grad_()
+        layer.layer_1.param_grad_is_zero = layer.layer_2.param_grad_is_zero = True
+        layer.router.grad = None
+        out = layer(x)
+        out.backward(grad_output)
+        return [t.clone() for t in (out.detach(), x.grad, layer.router.grad, layer.layer_1.grad_buffer,
+                                    layer.layer_2.grad_buffer)]  # fmt: skip
+
+    expected = [eager(x) for x in inputs]
+
+    static_input = inputs[0].clone().requires_grad_()
+    stream = torch.cuda.Stream(device=device)
+    stream.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(stream):
+        for _ in range(2):
+            layer.layer_1.param_grad_is_zero = layer.layer_2.param_grad_is_zero = True
+            layer(static_input).backward(grad_output)
+    torch.cuda.current_stream(device).wait_stream(stream)
+    torch.cuda.synchronize()
+    static_input.grad = None
+    layer.router.grad = None
+    layer.layer_1.param_grad_is_zero = layer.layer_2.param_grad_is_zero = True
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        static_output = layer(static_input)
+        static_output.backward(grad_output)
+    # The tensors the graph writes (eager work below rebinds `layer.router.grad`).
+    static_results = (static_output.detach(), static_input.grad, layer.router.grad, layer.layer_1.grad_buffer,
+                      layer.layer_2.grad_buffer)  # fmt: skip
+    for x, reference in zip(inputs + inputs, expected + expected):
+        static_input.data.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        results = [t.clone() for t in static_results]
+        for a, b in zip(results, reference):
+            assert torch.equal(a, b)
+        # eager work between replays (it overwrites the gradient buffers, which the next replay writes again)
+        assert all(torch.equal(a, b) for a, b in zip(eager(x), reference))
