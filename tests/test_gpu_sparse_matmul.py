@@ -344,3 +344,53 @@ def test_split_reduction_of_last_round(experts, inner, other, dtype, device):
     # dense product through the same kernel
     expected = (x.float() @ weight[:inner].float()).to(dtype)
     assert max_rel_err(dense_matmul(x_gpu, weight[:inner].to(device)).cpu(), expected) <= tolerance
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_through_the_matrix_core_kernel(seed, device):
+    """A sweep over ragged expert layouts and sizes around the kernel's tile (256 x 256 x 64), slice-pair and
+    split-reduction boundaries; all three products, random accumulation and output width."""
+    generator = torch.Generator().manual_seed(1000 + seed)
+
+    def pick(*choices):
+        return choices[int(torch.randint(0, len(choices), (1,), generator=generator))]
+
+    experts = pick(1, 3, 8, 20)
+    inner = pick(64, 128, 192, 448, 2048, 2112, 4160)
+    other = pick(8, 72, 256, 264, 520)
+    dtype = pick(torch.bfloat16, torch.float16)
+    case = _ragged_case(seed, experts)
+    oracle_map = fixture_sparse_map(case)
+    oracle_map.num_rows = case["expert_ends"][-1] + case["phantom_rows"]
+    sparse_map = to_device_map(oracle_map, device, pick(torch.int16, torch.int32, torch.int64))
+    used = _used_rows(oracle_map)
+    tolerance = _MAX_REL[dtype]
+    rows = oracle_map.num_rows
+    x = _normal(rows, inner, dtype, generator)
+    x[~oracle_map.real_row_mask()] = 0  # padding rows hold zeros here so that every product is finite
+    x_gpu = x.to(device)
+
+    # output-sparse
+    weight = _normal(experts * other, inner, dtype, generator)
+    out_dtype = pick(dtype, torch.float32)
+    accumulate = pick(False, True)
+    previous = _normal(rows, other, out_dtype, generator)
+    out = previous.to(device)
+    output_sparse_matmul(x_gpu, weight.to(device).t(), sparse_map, out, accumulate=accumulate)
+    expected = moe_oracle.output_sparse_matmul(x, weight.t(), oracle_map, out=previous.clone(), accumulate=accumulate)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+    assert torch.equal(out[used:].cpu(), previous[used:])
+
+    # input-inner-sparse
+    weight = _normal(experts * inner, other, dtype, generator)
+    out = input_inner_sparse_matmul(x_gpu, weight.to(device), sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(x, weight, oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+
+    # input-row-sparse: the reduction runs over the (ragged) rows
+    y = _normal(rows, other, dtype, generator)
+    out_dtype = pick(dtype, torch.float32)
+    out = torch.full((experts * inner, other), 2.0, dtype=out_dtype, device=device)
+    input_row_sparse_matmul(x_gpu.t(), y.to(device), sparse_map, out=out)
+    expected = moe_oracle.input_row_sparse_matmul(x.t(), y, oracle_map, out=torch.zeros(out.shape, dtype=out_dtype))
+    assert max_rel_err(out.cpu(), expected) <= tolerance
