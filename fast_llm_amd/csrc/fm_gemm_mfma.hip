@@ -503,9 +503,21 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
     const bool column_ok = column_in_tile < cols_valid;
     const int first_row = wave_m * kWaveRows + read_row;
     OutT *pointer = out + first_row * stride + column_in_tile;
+    const bool whole_tile = rows_valid == kTile && cols_valid == kTile;
 #pragma unroll
     for (int i = 0; i < kTilesM; ++i) {
         auto &&block = source(i);
+        // When adding to `out`: what it holds is requested first, all of the block's chunks at once, so that the
+        // loads are on their way while the accumulators go through LDS (loads issued one by one between the stores
+        // would each wait out a full memory latency: the compiler cannot move them across stores to the same array).
+        Vec16x4<OutT> previous[kAccumulate ? kReads : 1];
+        if constexpr (kAccumulate) {
+            const OutT *source_row = pointer + static_cast<int64_t>(i) * 32 * stride;
+#pragma unroll
+            for (int t = 0; t < kReads; ++t, source_row += kRowsPerRead * stride)
+                if (whole_tile || (first_row + i * 32 + t * kRowsPerRead < rows_valid && column_ok))
+                    previous[t] = *reinterpret_cast<const Vec16x4<OutT> *>(source_row);
+        }
 #pragma unroll
         for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
@@ -534,7 +546,7 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
                 }
                 if constexpr (kAccumulate) {
                     const f32x4_t value = __builtin_bit_cast(f32x4_t, staged[t]);
-                    Vec16x4<OutT> packed = *reinterpret_cast<const Vec16x4<OutT> *>(target);
+                    Vec16x4<OutT> packed = previous[t];
 #pragma unroll
                     for (int c = 0; c < 4; ++c) packed.v[c] = from_float<OutT>(value[c] + to_float(packed.v[c]));
                     store_streaming(target, packed);
@@ -543,7 +555,7 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
                 }
             }
         };
-        if (rows_valid == kTile && cols_valid == kTile) store_rows(std::true_type{});
+        if (whole_tile) store_rows(std::true_type{});
         else store_rows(std::false_type{});
         asm volatile("" ::: "memory");
     }
