@@ -3,7 +3,8 @@ Writes `tests/golden/golden_small.npz`: inputs and expected outputs of small cas
 
 Expected values do not come from the oracle's own formulas: the sparse map is computed by the brute-force O(M*E)
 python loops of `tests/helpers.py`, the MoE outputs and gradients by a token-by-token textbook mixture in float64
-differentiated by torch autograd. (The reference itself cannot be imported under this Python; see DESIGN.md.)
+differentiated by torch autograd. (The reference itself cannot be imported under this Python: it needs 3.12's
+PEP 695 generics and `enum.StrEnum`, fast_llm/utils.py:35, fast_llm/functional/config.py:31.)
 
 Run from the repository root: `python tests/golden/make_golden.py`.
 """
