@@ -26,8 +26,10 @@
 //   * The tile is written through LDS, already rounded to the output type, as 16-byte streaming stores that cover
 //     full 256-byte row segments.
 //   * Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are renumbered so that the tiles an XCD
-//     runs at the same time are 8 row tiles x 4 column tiles that re-read operands from its own L2.
-// Results are deterministic: one workgroup per output tile, fixed summation order, no atomics.
+//     runs at the same time are about 8 row tiles x 4 column tiles of one expert, which re-read operands from its L2.
+//   * When a launch has few rounds of long tiles, the reductions of the last round's tiles are split over the idle
+//     CUs and a second kernel adds the pieces in a fixed order.
+// Results are deterministic: one workgroup per output tile (or a fixed split), fixed summation order, no atomics.
 #include <type_traits>
 
 #include "fm_activation_math.h"
@@ -276,19 +278,55 @@ struct TileWork {
     int64_t k_lo, k_hi;
 };
 
-// The t-th 256-row tile over all experts, in expert order (expert e contributes ceil(rows_e / 256) tiles).
-// Every wavefront scans `expert_ends` 64 experts at a time; returns false if there are fewer than t + 1 tiles.
-__device__ __forceinline__ bool find_row_tile(const GemmArgs &args, int tile, int &expert, int64_t &row0,
-                                              int &rows_valid) {
+constexpr int kXcds = 8, kGroupRows = 8, kChunkTiles = 32;
+
+// Logical order of the tiles of a product whose rows are grouped by expert (output-sparse, input-inner-sparse,
+// dense): expert after expert; within an expert its row tiles (ceil(rows_e / 256)) are cut into ceil(count / 8)
+// groups of nearly equal size (9 row tiles: 5 + 4), and a group is walked column tile by column tile, row tiles
+// fastest. 32 consecutive tiles (what an XCD runs at one time) are then about 8 row tiles x 4 column tiles of ONE
+// expert, i.e. 8 lhs panels and 4 rhs panels shared in that XCD's L2; with groups that ignore the expert boundaries
+// most chunks straddled two experts and needed twice the rhs panels.
+// Every wavefront scans `expert_ends` 64 experts at a time; returns false if `logical` is past the last tile.
+struct RowTile {
+    int expert, tile_n, rows_valid;
+    int64_t row0;
+};
+
+__device__ __forceinline__ void place_in_expert(int local, int count, int tiles_n, int &row_tile, int &tile_n) {
+    const int groups = (count + kGroupRows - 1) / kGroupRows;
+    const int base = count / groups, larger = count % groups;  // the first `larger` groups have base + 1 row tiles
+    const int larger_tiles = larger * (base + 1) * tiles_n;
+    int first_row, rows, in_group;
+    if (local < larger_tiles) {
+        const int group = local / ((base + 1) * tiles_n);
+        rows = base + 1;
+        first_row = group * rows;
+        in_group = local - group * rows * tiles_n;
+    } else {
+        const int rest = local - larger_tiles;
+        const int group = rest / (base * tiles_n);
+        rows = base;
+        first_row = larger * (base + 1) + group * rows;
+        in_group = rest - group * rows * tiles_n;
+    }
+    row_tile = first_row + in_group % rows;
+    tile_n = in_group / rows;
+}
+
+__device__ __forceinline__ bool locate_tile(const GemmArgs &args, int logical, RowTile &tile) {
+    const int tiles_n = args.tiles_n;
     if (args.expert_ends == nullptr) {
-        expert = 0;
-        row0 = static_cast<int64_t>(tile) * kTile;
-        if (row0 >= args.rows) return false;
-        rows_valid = static_cast<int>(min(static_cast<int64_t>(kTile), args.rows - row0));
+        const int count = static_cast<int>((args.rows + kTile - 1) / kTile);
+        if (logical >= count * tiles_n) return false;
+        int row_tile;
+        place_in_expert(logical, count, tiles_n, row_tile, tile.tile_n);
+        tile.expert = 0;
+        tile.row0 = static_cast<int64_t>(row_tile) * kTile;
+        tile.rows_valid = static_cast<int>(min(static_cast<int64_t>(kTile), args.rows - tile.row0));
         return true;
     }
     const int lane = threadIdx.x & 63;
-    int tiles_before = 0;
+    int tiles_before = 0;  // row tiles of the experts before this block of 64
     for (int base = 0; base < args.num_experts; base += 64) {
         const int e = base + lane;
         int64_t begin = 0, end = 0;
@@ -304,14 +342,17 @@ __device__ __forceinline__ bool find_row_tile(const GemmArgs &args, int tile, in
             if (lane >= offset) inclusive += other;
         }
         const int total = __shfl(inclusive, 63, 64);
-        if (tile < tiles_before + total) {
-            const uint64_t owners = __ballot(tiles_before + inclusive > tile);
+        if (logical < (tiles_before + total) * tiles_n) {
+            const uint64_t owners = __ballot((tiles_before + inclusive) * tiles_n > logical);
             const int owner = __ffsll(static_cast<unsigned long long>(owners)) - 1;
+            const int owner_count = __shfl(count, owner, 64);
             const int first_tile = tiles_before + __shfl(inclusive - count, owner, 64);
             const int64_t owner_begin = __shfl(begin, owner, 64), owner_end = __shfl(end, owner, 64);
-            expert = base + owner;
-            row0 = owner_begin + static_cast<int64_t>(tile - first_tile) * kTile;
-            rows_valid = static_cast<int>(min(static_cast<int64_t>(kTile), owner_end - row0));
+            int row_tile;
+            place_in_expert(logical - first_tile * tiles_n, owner_count, tiles_n, row_tile, tile.tile_n);
+            tile.expert = base + owner;
+            tile.row0 = owner_begin + static_cast<int64_t>(row_tile) * kTile;
+            tile.rows_valid = static_cast<int>(min(static_cast<int64_t>(kTile), owner_end - tile.row0));
             return true;
         }
         tiles_before += total;
@@ -319,15 +360,29 @@ __device__ __forceinline__ bool find_row_tile(const GemmArgs &args, int tile, in
     return false;
 }
 
-__device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int tile_m, int tile_n, TileWork &work) {
-    // A tile of the fused gated forward product has 128 gate columns (and their up columns).
-    const bool paired = args.fusion == kFusionGatedForward;
-    const int64_t col0 = static_cast<int64_t>(tile_n) * (paired ? kTile / 2 : kTile);
-    work.cols_valid = paired ? kTile : static_cast<int>(min(static_cast<int64_t>(kTile), args.cols - col0));
-    work.fused_offset = 0;
+// Logical tile -> (row tile, column tile) for the row-sparse product, whose row tiles are expert-aligned by
+// construction: groups of 8 row tiles, column by column inside a group.
+__device__ __forceinline__ void tile_coordinates(int logical, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
+    const int width = kGroupRows * tiles_n;
+    const int group = logical / width;
+    const int first_m = group * kGroupRows;
+    const int group_rows = min(tiles_m - first_m, kGroupRows);
+    const int in_group = logical - group * width;
+    tile_m = first_m + in_group % group_rows;
+    tile_n = in_group / group_rows;
+}
+
+// Where the operands and the output of logical tile `logical` are. False: there is no such tile.
+__device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int logical, TileWork &work) {
     work.k_lo = 0;
     work.k_hi = args.inner;
+    work.fused_offset = 0;
     if (args.mode == kInputRowSparse) {
+        if (logical >= args.tiles_m * args.tiles_n) return false;
+        int tile_m, tile_n;
+        tile_coordinates(logical, args.tiles_m, args.tiles_n, tile_m, tile_n);
+        const int64_t col0 = static_cast<int64_t>(tile_n) * kTile;
+        work.cols_valid = static_cast<int>(min(static_cast<int64_t>(kTile), args.cols - col0));
         const int tiles_per_expert = static_cast<int>((args.sparse_size + kTile - 1) / kTile);
         const int expert = tile_m / tiles_per_expert;
         const int64_t row_in_expert = static_cast<int64_t>(tile_m - expert * tiles_per_expert) * kTile;
@@ -343,17 +398,21 @@ __device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int tile_m, i
         work.out_offset = (expert * args.sparse_size + row_in_expert) * args.out_stride_row + col0;
         return true;
     }
-    int expert;
-    int64_t row0;
-    if (!find_row_tile(args, tile_m, expert, row0, work.rows_valid)) return false;
-    work.lhs_offset = row0 * args.lhs_stride_row;
-    work.out_offset = row0 * args.out_stride_row + col0;
-    work.fused_offset = row0 * args.fused_stride + col0;
+    RowTile tile;
+    if (!locate_tile(args, logical, tile)) return false;
+    // A tile of the fused gated forward product has 128 gate columns (and their up columns).
+    const bool paired = args.fusion == kFusionGatedForward;
+    const int64_t col0 = static_cast<int64_t>(tile.tile_n) * (paired ? kTile / 2 : kTile);
+    work.cols_valid = paired ? kTile : static_cast<int>(min(static_cast<int64_t>(kTile), args.cols - col0));
+    work.rows_valid = tile.rows_valid;
+    work.lhs_offset = tile.row0 * args.lhs_stride_row;
+    work.out_offset = tile.row0 * args.out_stride_row + col0;
+    work.fused_offset = tile.row0 * args.fused_stride + col0;
     if (args.mode == kOutputSparse)
-        work.rhs_offset = (static_cast<int64_t>(expert) * args.sparse_size + col0) * args.rhs_stride_col;
+        work.rhs_offset = (static_cast<int64_t>(tile.expert) * args.sparse_size + col0) * args.rhs_stride_col;
     else
         work.rhs_offset =
-            static_cast<int64_t>(expert) * args.sparse_size * args.rhs_stride_inner + col0 * args.rhs_stride_col;
+            static_cast<int64_t>(tile.expert) * args.sparse_size * args.rhs_stride_inner + col0 * args.rhs_stride_col;
     return true;
 }
 
@@ -363,22 +422,10 @@ __device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int tile_m, i
 // chunk, i.e. 8 row tiles x 4 column tiles that share operand panels in that XCD's L2, while consecutive chunks go to
 // different XCDs, so that experts with many and with few tokens (long and short tiles of the row-sparse product)
 // are spread over all of them. A permutation of every aligned block of 256 ids.
-constexpr int kXcds = 8, kGroupRows = 8, kChunkTiles = 32;
 constexpr int kRound = kXcds * kChunkTiles;  // workgroups that run at the same time: one per CU
 __device__ __forceinline__ int logical_of_block(int pid) {
     const int xcd = pid % kXcds, local = pid / kXcds;
     return ((local / kChunkTiles) * kXcds + xcd) * kChunkTiles + local % kChunkTiles;
-}
-
-// Logical tile -> (row tile, column tile): groups of 8 row tiles, column by column inside a group.
-__device__ __forceinline__ void tile_coordinates(int logical, int tiles_m, int tiles_n, int &tile_m, int &tile_n) {
-    const int width = kGroupRows * tiles_n;
-    const int group = logical / width;
-    const int first_m = group * kGroupRows;
-    const int group_rows = min(tiles_m - first_m, kGroupRows);
-    const int in_group = logical - group * width;
-    tile_m = first_m + in_group % group_rows;
-    tile_n = in_group / group_rows;
 }
 
 // ---- splitting the reduction of the last tiles ---------------------------------------------------------------
@@ -448,19 +495,15 @@ __device__ __forceinline__ SplitPlan plan_split(const GemmArgs &args) {
     return plan;
 }
 
-// What the workgroup `pid` of the main kernel computes. Without a workspace (piece_slot < 0 on return) the row tile
-// count is the host's upper bound and ids past the tiles that exist are weeded out later, by resolve_tile.
-__device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int &tile_m, int &tile_n, int &piece,
+// The logical tile the workgroup `pid` of the main kernel computes, whole (piece_slot < 0) or as piece `piece` of a
+// split reduction. Without a workspace, ids past the tiles that exist are weeded out later, by resolve_tile.
+__device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int &logical, int &piece,
                                               int &piece_slices, int &piece_slot) {
-    int logical = logical_of_block(pid);
+    logical = logical_of_block(pid);
     piece = 0;
     piece_slices = 0;
     piece_slot = -1;
-    if (args.partials == nullptr) {
-        if (logical >= args.tiles_m * args.tiles_n) return false;
-        tile_coordinates(logical, args.tiles_m, args.tiles_n, tile_m, tile_n);
-        return true;
-    }
+    if (args.partials == nullptr) return true;
     const SplitPlan plan = plan_split(args);
     if (logical >= plan.whole) {
         const int index = logical - plan.whole;
@@ -472,7 +515,6 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int
             logical = plan.whole + index - piece * plan.tail;
         }
     }
-    tile_coordinates(logical, plan.tiles_m, args.tiles_n, tile_m, tile_n);
     return true;
 }
 
@@ -753,10 +795,9 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);  // C-style: address-space cast
 
-    int tile_m, tile_n, piece, piece_slices, piece_slot;
+    int logical, piece, piece_slices, piece_slot;
     TileWork work;
-    if (!tile_of_block(args, blockIdx.x, tile_m, tile_n, piece, piece_slices, piece_slot) ||
-        !resolve_tile(args, tile_m, tile_n, work))
+    if (!tile_of_block(args, blockIdx.x, logical, piece, piece_slices, piece_slot) || !resolve_tile(args, logical, work))
         return;
     piece_slot = __builtin_amdgcn_readfirstlane(piece_slot);
     if (piece_slot >= 0) {  // a piece of a tile whose reduction is split (never the row-sparse product)
@@ -966,10 +1007,8 @@ __global__ __launch_bounds__(64) void grouped_gemm_reduce_kernel(GemmArgs args) 
     const SplitPlan plan = plan_split(args);
     const int index = blockIdx.x / kWaves;
     if (plan.pieces == 1 || index >= plan.tail) return;
-    int tile_m, tile_n;
     TileWork work;
-    tile_coordinates(plan.whole + index, plan.tiles_m, args.tiles_n, tile_m, tile_n);
-    if (!resolve_tile(args, tile_m, tile_n, work)) return;
+    if (!resolve_tile(args, plan.whole + index, work)) return;
     const int lane = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x % kWaves));
     // One block of 32 rows at a time: 64 registers of sums, the loads of a piece all in flight together.
