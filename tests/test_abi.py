@@ -62,6 +62,45 @@ def test_argument_validation_returns_status_and_message(library):
     assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"dtype" in library.fm_last_error()
 
 
+def test_router_and_fused_entry_points_validate_before_launching(library):
+    assert library.fm_router_workspace_size(8192, 8) >= 4 * (2 * 8 + 1)
+    assert library.fm_router_workspace_size(0, 8) == 0
+    fake = 256  # a non-null "pointer" that validation must never dereference
+    args = dict(tokens=16, experts=8, k=2, shared=0)
+
+    def forward(workspace_size=1 << 20, dtype=0, **overrides):
+        a = {**args, **overrides}
+        return library.fm_router_forward(fake, None, fake, fake, fake, fake, fake, fake, workspace_size, a["tokens"],
+                                         a["experts"], a["k"], a["shared"], dtype, None)  # fmt: skip
+
+    assert forward(experts=2000) == _lib.FM_ERR_INVALID_ARGUMENT and b"experts" in library.fm_last_error()
+    assert forward(k=60, shared=10, experts=64) == _lib.FM_ERR_INVALID_ARGUMENT
+    assert forward(k=9) == _lib.FM_ERR_INVALID_ARGUMENT and b"experts_per_token" in library.fm_last_error()
+    assert forward(workspace_size=8) == _lib.FM_ERR_INVALID_ARGUMENT and b"workspace" in library.fm_last_error()
+    assert forward(dtype=9) == _lib.FM_ERR_INVALID_ARGUMENT
+    status = library.fm_router_backward(fake, fake, fake, fake, None, fake, fake, None, 0.0, 0.0, 16, 8, 2, 0, 0, None)
+    assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"null" in library.fm_last_error()
+
+    # The fused products exist for the matrix-core kernel only: anything else is reported, not emulated.
+    def fused(dtype=1, activation_dim=256, inner=128, activation=1, lhs_stride_inner=1):
+        return library.fm_output_sparse_matmul_gated_activation(
+            fake, fake, fake, fake, None, 256, activation_dim, inner, 1, inner, lhs_stride_inner, 1, inner, activation,
+            dtype, 1, None,
+        )  # fmt: skip
+
+    assert fused(dtype=0) == _lib.FM_ERR_UNSUPPORTED and b"separately" in library.fm_last_error()
+    with pytest.raises(NotImplementedError):
+        _lib.check(_lib.FM_ERR_UNSUPPORTED)
+    assert fused(activation_dim=200) == _lib.FM_ERR_UNSUPPORTED  # not a multiple of 128
+    assert fused(inner=100) == _lib.FM_ERR_UNSUPPORTED  # reduction not in whole 64-element slices
+    assert fused(lhs_stride_inner=2) == _lib.FM_ERR_UNSUPPORTED
+    assert fused(activation=42) == _lib.FM_ERR_INVALID_ARGUMENT and b"activation" in library.fm_last_error()
+    status = library.fm_output_sparse_matmul_gated_activation_backward(
+        fake, fake, None, fake, None, None, 256, 256, 128, 1, 128, 1, 1, 128, 1, 1, 1, None
+    )
+    assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"null" in library.fm_last_error()
+
+
 def test_cpu_tensors_are_refused_not_emulated(library):
     top_experts = torch.zeros(4, 2, dtype=torch.int64)
     with pytest.raises(RuntimeError, match="GPU"):
