@@ -35,6 +35,7 @@
 #include "fm_activation_math.h"
 #include "fm_gemm_common.h"
 
+#include <atomic>
 #include <mutex>
 #include <stdlib.h>
 
@@ -1042,33 +1043,34 @@ __global__ __launch_bounds__(64) void grouped_gemm_reduce_kernel(GemmArgs args) 
 }
 
 // ---- host side -----------------------------------------------------------------------------------------
-static int allow_big_lds(const void *kernel) {
-    hipError_t error = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+// Kernels that use more dynamic LDS than the default limit need the attribute set once per device; `configured` is the
+// kernel's own bit mask of devices done (setting it twice from racing threads is harmless).
+static int allow_lds(const void *kernel, int bytes, std::atomic<uint64_t> &configured) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return fail(FM_ERR_LAUNCH, "hipGetDevice failed");
+    const uint64_t bit = uint64_t(1) << (device & 63);
+    if (device < 64 && (configured.load(std::memory_order_relaxed) & bit)) return FM_OK;
+    hipError_t error = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
+    if (device < 64) configured.fetch_or(bit, std::memory_order_relaxed);
     return FM_OK;
 }
 
 template <typename T, bool kLhsK, bool kRhsK, bool kMasked, int kFusion = kFusionNone>
 static int launch_instance(const GemmArgs &args, hipStream_t stream) {
     auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK, kMasked, kFusion>;
-    static bool configured = false;  // setting the attribute twice from racing threads is harmless
-    if (!configured) {
-        if (int status = allow_big_lds(reinterpret_cast<const void *>(kernel))) return status;
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int status = allow_lds(reinterpret_cast<const void *>(kernel), kLdsBytes, configured)) return status;
     // Whole rounds of one chunk per XCD; the surplus workgroups find no tile and exit. With a workspace the pieces
     // of the last round's tiles come after the whole tiles, at most kMaxPartials of them.
     int grid = (args.tiles_m * args.tiles_n + kRound - 1) / kRound * kRound;
     if (args.partials != nullptr) grid += kMaxPartials;
     kernel<<<grid, kMfmaThreads, kLdsBytes, stream>>>(args);
     if (args.partials != nullptr) {
-        static bool reduce_configured = false;
-        if (!reduce_configured) {
-            hipError_t error = hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_reduce_kernel),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kReduceLdsBytes);
-            if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
-            reduce_configured = true;
-        }
+        static std::atomic<uint64_t> reduce_configured{0};
+        if (int status = allow_lds(reinterpret_cast<const void *>(grouped_gemm_reduce_kernel), kReduceLdsBytes,
+                                   reduce_configured))
+            return status;
         grouped_gemm_reduce_kernel<<<kRound * kWaves, 64, kReduceLdsBytes, stream>>>(args);
     }
     return FM_OK;
