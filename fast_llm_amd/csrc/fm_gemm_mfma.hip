@@ -547,19 +547,28 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
     const int first_row = wave_m * kWaveRows + read_row;
     OutT *pointer = out + first_row * stride + column_in_tile;
     const bool whole_tile = rows_valid == kTile && cols_valid == kTile;
+    constexpr bool kAhead = sizeof(OutT) == 2;
+    Vec16x4<OutT> previous[kAccumulate && kAhead ? 2 : 1][kAccumulate ? kReads : 1];
+    auto load_previous = [&](int i, Vec16x4<OutT>(&values)[kAccumulate ? kReads : 1]) {
+        const OutT *source_row = pointer + static_cast<int64_t>(i) * 32 * stride;
+#pragma unroll
+        for (int t = 0; t < kReads; ++t, source_row += kRowsPerRead * stride)
+            if (whole_tile || (first_row + i * 32 + t * kRowsPerRead < rows_valid && column_ok))
+                values[t] = *reinterpret_cast<const Vec16x4<OutT> *>(source_row);
+    };
 #pragma unroll
     for (int i = 0; i < kTilesM; ++i) {
         auto &&block = source(i);
-        // When adding to `out`: what it holds is requested first, all of the block's chunks at once, so that the
-        // loads are on their way while the accumulators go through LDS (loads issued one by one between the stores
-        // would each wait out a full memory latency: the compiler cannot move them across stores to the same array).
-        Vec16x4<OutT> previous[kAccumulate ? kReads : 1];
-        if constexpr (kAccumulate) {
-            const OutT *source_row = pointer + static_cast<int64_t>(i) * 32 * stride;
-#pragma unroll
-            for (int t = 0; t < kReads; ++t, source_row += kRowsPerRead * stride)
-                if (whole_tile || (first_row + i * 32 + t * kRowsPerRead < rows_valid && column_ok))
-                    previous[t] = *reinterpret_cast<const Vec16x4<OutT> *>(source_row);
+        // When adding to `out`: what it holds is requested ahead of time, all chunks of a row block at once and one
+        // block ahead of the block being staged, so that the loads are on their way while accumulators go through
+        // LDS (loads issued one by one between the stores would each wait out a full memory latency: the compiler
+        // cannot move them across stores to the same array).
+        // (One block ahead only where the values are two bytes wide: two blocks of fp32 do not fit the registers.)
+        if constexpr (kAccumulate && kAhead) {
+            if (i == 0) load_previous(0, previous[0]);
+            if (i + 1 < kTilesM) load_previous(i + 1, previous[(i + 1) & 1]);
+        } else if constexpr (kAccumulate) {
+            load_previous(i, previous[0]);
         }
 #pragma unroll
         for (int j = 0; j < kTilesN; ++j)
@@ -589,7 +598,7 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
                 }
                 if constexpr (kAccumulate) {
                     const f32x4_t value = __builtin_bit_cast(f32x4_t, staged[t]);
-                    Vec16x4<OutT> packed = previous[t];
+                    Vec16x4<OutT> packed = previous[kAhead ? i & 1 : 0][t];
 #pragma unroll
                     for (int c = 0; c < 4; ++c) packed.v[c] = from_float<OutT>(value[c] + to_float(packed.v[c]));
                     store_streaming(target, packed);
