@@ -207,3 +207,30 @@ def test_layer_with_shared_experts_and_trained_router_losses(device):
     assert close(x.grad, x_cpu.grad)
     assert close(layer.router.grad, router_weight.grad)
     assert close(layer.layer_1.grad_buffer, weight_1.grad) and close(layer.layer_2.grad_buffer, weight_2.grad)
+
+
+def test_router_with_masked_experts_and_full_selection(device):
+    """Experts masked out with -inf logits (how the forced-empty benchmark case is built) are never selected, get
+    probability 0 and a zero gradient; with k equal to the number of experts every expert is selected and the scores
+    are the full softmax."""
+    generator = torch.Generator().manual_seed(8)
+    logits = torch.randn(300, 8, generator=generator)
+    logits[:, 5] = float("-inf")
+    leaf = logits.clone().requires_grad_()
+    expected = moe_oracle.router(leaf, 2)
+    grad_scores = torch.randn(300, 2, generator=generator)
+    expected_grad = moe_oracle.router_backward(expected, leaf, grad_scores, 0.3, 0.1)
+    gpu_logits = logits.to(device).requires_grad_()
+    scores, top_experts, load_balancing_loss, z_loss = router(gpu_logits, 2, auxiliary_loss_grad=0.3, z_loss_grad=0.1)
+    assert torch.equal(top_experts.cpu(), expected.top_experts) and not (top_experts == 5).any()
+    assert load_balancing_loss.item() == pytest.approx(expected.load_balancing_loss.item(), rel=1e-5)
+    assert z_loss.item() == pytest.approx(expected.z_loss.item(), rel=1e-5)
+    scores.backward(grad_scores.to(device))
+    assert torch.isfinite(gpu_logits.grad).all() and (gpu_logits.grad[:, 5] == 0).all()
+    assert torch.allclose(gpu_logits.grad.cpu(), expected_grad, rtol=1e-4, atol=1e-7)
+
+    logits = torch.randn(64, 6, generator=generator)
+    scores, top_experts, _, _ = router(logits.to(device), 6)
+    assert torch.equal(top_experts.cpu().sort(dim=-1).values, torch.arange(6).expand(64, 6))
+    full = torch.softmax(logits, dim=-1)
+    assert torch.allclose(scores.cpu(), full.gather(1, top_experts.cpu()), rtol=2e-6, atol=1e-7)
