@@ -4,7 +4,12 @@
  * Every entry point
  *   - takes plain device pointers, 64-bit sizes/strides (in elements) and small integer enums;
  *   - launches asynchronously on the HIP stream passed last (`void *` holding a `hipStream_t`, NULL = default
- *     stream) and never synchronises, allocates or frees device memory, or keeps a pointer after it returns;
+ *     stream) and never synchronises, frees device memory, or keeps a caller's pointer after it returns. It does
+ *     not allocate either, with one exception: the three grouped products keep a workspace of 128 MiB per
+ *     (device, stream) for splitting the reductions of a launch's last tiles over idle CUs; it is allocated at a
+ *     stream's first product with few tiles and a long reduction (never while the stream is being captured: the
+ *     product then runs unsplit) and kept until the process ends. FASTMOE_SPLIT_REDUCTION=0 in the environment
+ *     turns the split, and with it the allocation, off;
  *   - returns `FM_OK` (0) or a negative `fm_status`; the message for the calling thread is read with
  *     `fm_last_error()`. No C++ exception crosses this boundary.
  *
