@@ -92,6 +92,8 @@ _ROUTER_CASES = [
     (300, 130, 8, 3, False),
     (5, 1000, 60, 4, False),
     (1, 2, 1, 0, True),
+    (16384, 128, 8, 0, False),  # the routers of the wide and fine-grained configurations at full size
+    (16384, 64, 6, 2, False),
 ]
 
 
