@@ -47,6 +47,13 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--cpu-tokens", type=int, default=8192, help="tokens in the CPU baseline sample (0: skip)")
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument(
+        "--grad-dtype",
+        default="same",
+        choices=("same", "fp32"),
+        help="dtype of the weight-gradient buffers: the weights' own (what the reference's kernel benchmarks and "
+        "functional tests attach: torch.empty_like(param)) or float32 (the training engine's full_precision_gradients)",
+    )
+    parser.add_argument(
         "--calibration-mib",
         type=int,
         default=1024,
@@ -113,8 +120,9 @@ def main() -> None:
     inputs = make_inputs(workload, seed=args.seed, weight_device=device).to(device)
     x = inputs.hidden_states.requires_grad_(True)
     scores = inputs.scores.requires_grad_(True)
-    weight_1 = attach_grad_buffer(inputs.weight_1.requires_grad_(True))
-    weight_2 = attach_grad_buffer(inputs.weight_2.requires_grad_(True))
+    grad_dtype = torch.float32 if args.grad_dtype == "fp32" else None
+    weight_1 = attach_grad_buffer(inputs.weight_1.requires_grad_(True), grad_dtype)
+    weight_2 = attach_grad_buffer(inputs.weight_2.requires_grad_(True), grad_dtype)
 
     def step() -> None:
         x.grad = scores.grad = None
