@@ -150,19 +150,20 @@ __global__ __launch_bounds__(kGenThreads) void grouped_gemm_generic_kernel(GemmA
 // =========================================================================================================
 // Host dispatch
 // =========================================================================================================
-static int run_gemm(const char *name, GemmArgs args, int dtype, void *stream_) {
+static int run_gemm(const char *name, GemmArgs args, int dtype, void *workspace, size_t workspace_size, void *stream_) {
     FM_REQUIRE(valid_dtype(dtype) && valid_dtype(args.out_dtype), "%s: bad dtype", name);
     FM_REQUIRE(valid_index_dtype(args.index_dtype), "%s: bad index_dtype %d", name, args.index_dtype);
     FM_REQUIRE(args.rows >= 0 && args.cols >= 0 && args.inner >= 0 && args.sparse_size >= 0 && args.num_experts >= 1,
                "%s: negative shape", name);
     FM_REQUIRE(args.mode != kInputRowSparse || args.expert_ends == nullptr || args.expert_pad_begins != nullptr,
                "%s: null expert_pad_begins", name);
+    FM_REQUIRE(workspace != nullptr || workspace_size == 0, "%s: null workspace of %zu bytes", name, workspace_size);
     if (args.rows == 0 || args.cols == 0) return FM_OK;
     FM_REQUIRE(args.out && (args.inner == 0 || (args.lhs && args.rhs)), "%s: null tensor", name);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
 
     if (mfma_gemm_eligible(args, dtype)) {
-        if (int status = mfma_gemm_launch(args, dtype, stream)) return status;
+        if (int status = mfma_gemm_launch(args, dtype, workspace, workspace_size, stream)) return status;
     } else {
         // A row-sparse tile must not cross into the next expert's block of out.
         if (args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % kGenTile != 0)
@@ -185,12 +186,13 @@ extern "C" int fm_output_sparse_matmul(const void *lhs, const void *rhs, void *o
                                        int64_t row_dim, int64_t col_sparse_dim, int64_t inner_dim, int64_t num_experts,
                                        int64_t lhs_stride_row, int64_t lhs_stride_inner, int64_t rhs_stride_inner,
                                        int64_t rhs_stride_col, int64_t out_stride_row, int64_t out_stride_col,
-                                       int accumulate, int dtype, int out_dtype, int index_dtype, void *stream) {
+                                       int accumulate, int dtype, int out_dtype, int index_dtype, void *workspace,
+                                       size_t workspace_size, void *stream) {
     GemmArgs args{lhs, rhs, out, expert_ends, nullptr, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
                   rhs_stride_col, out_stride_row, out_stride_col, row_dim, col_sparse_dim, inner_dim, col_sparse_dim,
                   static_cast<int>(expert_ends ? num_experts : 1), kOutputSparse, accumulate, index_dtype, out_dtype, 0, 0, nullptr};
     FM_REQUIRE(num_experts >= 1 && num_experts < (1 << 20), "fm_output_sparse_matmul: bad num_experts");
-    return run_gemm("fm_output_sparse_matmul", args, dtype, stream);
+    return run_gemm("fm_output_sparse_matmul", args, dtype, workspace, workspace_size, stream);
 }
 
 extern "C" int fm_input_inner_sparse_matmul(const void *lhs, const void *rhs, void *out, const void *expert_ends,
@@ -198,12 +200,12 @@ extern "C" int fm_input_inner_sparse_matmul(const void *lhs, const void *rhs, vo
                                             int64_t num_experts, int64_t lhs_stride_row, int64_t lhs_stride_inner,
                                             int64_t rhs_stride_inner, int64_t rhs_stride_col, int64_t out_stride_row,
                                             int64_t out_stride_col, int accumulate, int dtype, int out_dtype,
-                                            int index_dtype, void *stream) {
+                                            int index_dtype, void *workspace, size_t workspace_size, void *stream) {
     GemmArgs args{lhs, rhs, out, expert_ends, nullptr, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
                   rhs_stride_col, out_stride_row, out_stride_col, row_dim, col_dim, inner_sparse_dim, inner_sparse_dim,
                   static_cast<int>(expert_ends ? num_experts : 1), kInputInnerSparse, accumulate, index_dtype, out_dtype, 0, 0, nullptr};
     FM_REQUIRE(num_experts >= 1 && num_experts < (1 << 20), "fm_input_inner_sparse_matmul: bad num_experts");
-    return run_gemm("fm_input_inner_sparse_matmul", args, dtype, stream);
+    return run_gemm("fm_input_inner_sparse_matmul", args, dtype, workspace, workspace_size, stream);
 }
 
 extern "C" int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void *out, const void *expert_ends,
@@ -211,13 +213,27 @@ extern "C" int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void
                                           int64_t inner_dim, int64_t num_experts, int64_t lhs_stride_row,
                                           int64_t lhs_stride_inner, int64_t rhs_stride_inner, int64_t rhs_stride_col,
                                           int64_t out_stride_row, int64_t out_stride_col, int accumulate, int dtype,
-                                          int out_dtype, int index_dtype, void *stream) {
+                                          int out_dtype, int index_dtype, void *workspace, size_t workspace_size,
+                                          void *stream) {
     FM_REQUIRE(num_experts >= 1 && num_experts < (1 << 20), "fm_input_row_sparse_matmul: bad num_experts");
     const int64_t experts = expert_ends ? num_experts : 1;
     GemmArgs args{lhs, rhs, out, expert_ends, expert_pad_begins, lhs_stride_row, lhs_stride_inner, rhs_stride_inner,
                   rhs_stride_col, out_stride_row, out_stride_col, row_sparse_dim * experts, col_dim, inner_dim,
                   row_sparse_dim, static_cast<int>(experts), kInputRowSparse, accumulate, index_dtype, out_dtype, 0, 0, nullptr};
-    return run_gemm("fm_input_row_sparse_matmul", args, dtype, stream);
+    return run_gemm("fm_input_row_sparse_matmul", args, dtype, workspace, workspace_size, stream);
+}
+
+extern "C" size_t fm_grouped_gemm_workspace_size(int64_t row_dim, int64_t col_dim, int64_t inner_dim,
+                                                 int64_t num_experts, int dtype) {
+    if (dtype != FM_DTYPE_BF16 && dtype != FM_DTYPE_F16) return 0;  // fp32 operands never take the splitting kernel
+    if (row_dim <= 0 || col_dim <= 0 || inner_dim <= 0 || num_experts < 0 || num_experts >= (1 << 20)) return 0;
+    GemmArgs args{};
+    args.rows = row_dim;
+    args.cols = col_dim;
+    args.inner = inner_dim;
+    args.num_experts = static_cast<int>(num_experts > 1 ? num_experts : 1);
+    args.mode = kOutputSparse;  // the input-inner-sparse product tiles the same way
+    return mfma_gemm_workspace_size(args);
 }
 
 // ---- grouped products with the gated activation fused into the epilogue ------------------------------------
@@ -236,7 +252,7 @@ static int run_fused_gemm(const char *name, GemmArgs args, int dtype, void *stre
                     "width that is a multiple of 128 (forward) or 8 (backward); run the product and the activation "
                     "separately",
                     name);
-    if (int status = mfma_gemm_launch(args, dtype, static_cast<hipStream_t>(stream))) return status;
+    if (int status = mfma_gemm_launch(args, dtype, nullptr, 0, static_cast<hipStream_t>(stream))) return status;
     return check_launch(name);
 }
 

@@ -33,7 +33,7 @@ struct GemmArgs {
     int index_dtype;
     int out_dtype;
     int tiles_m, tiles_n;
-    float *partials;  // workspace of the MFMA kernel for split reductions, or null; set by its launcher
+    float *partials;  // the caller's workspace when the MFMA kernel splits reductions, else null; set by its launcher
     int fusion;       // GemmFusion
     int activation;   // fm_activation tag, for the fused epilogues
     const void *fused_in;
@@ -59,6 +59,8 @@ __device__ __forceinline__ void store_out_dyn(void *out, int out_dtype, int64_t 
 // `args` (with `dtype` operands); `launch` fills in the tile counts and launches it.
 bool mfma_gemm_eligible(const GemmArgs &args, int dtype);
 bool mfma_gemm_fusion_eligible(const GemmArgs &args, int dtype);  // with args.fusion set
-int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream);
+// `workspace` (may be null: no split) must hold mfma_gemm_workspace_size(args) bytes when that is not 0.
+size_t mfma_gemm_workspace_size(GemmArgs args);
+int mfma_gemm_launch(GemmArgs args, int dtype, void *workspace, size_t workspace_size, hipStream_t stream);
 
 }  // namespace fm

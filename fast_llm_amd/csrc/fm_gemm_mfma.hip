@@ -27,8 +27,8 @@
 //     full 256-byte row segments.
 //   * Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are renumbered so that the tiles an XCD
 //     runs at the same time are about 8 row tiles x 4 column tiles of one expert, which re-read operands from its L2.
-//   * When a launch has few rounds of long tiles, the reductions of the last round's tiles are split over the idle
-//     CUs and a second kernel adds the pieces in a fixed order.
+//   * When a launch has few rounds of long tiles and the caller brings a workspace, the reductions of the last
+//     round's tiles are split over the idle CUs and a second kernel adds the pieces in a fixed order.
 // Results are deterministic: one workgroup per output tile (or a fixed split), fixed summation order, no atomics.
 #include <type_traits>
 
@@ -36,8 +36,6 @@
 #include "fm_gemm_common.h"
 
 #include <atomic>
-#include <mutex>
-#include <stdlib.h>
 
 namespace fm {
 
@@ -1123,53 +1121,6 @@ bool mfma_gemm_eligible(const GemmArgs &args, int dtype) {
     return true;
 }
 
-// ---- workspace for split reductions --------------------------------------------------------------------
-// kMaxPartials tiles of fp32 (128 MiB) per (device, stream) that has needed one, allocated at the first such call and
-// kept until the process ends. Kernels on one stream run in order, so calls on one stream can share a workspace;
-// calls on different streams may overlap and get their own.
-namespace {
-struct Workspace {
-    int device;
-    hipStream_t stream;
-    float *pointer;
-};
-constexpr int kMaxWorkspaces = 16;
-Workspace workspaces[kMaxWorkspaces];
-int num_workspaces = 0;
-std::mutex workspace_mutex;
-
-bool split_enabled() {
-    static const bool enabled = [] {
-        const char *value = getenv("FASTMOE_SPLIT_REDUCTION");
-        return value == nullptr || value[0] != '0';
-    }();
-    return enabled;
-}
-
-// Null when there is none and none can be had (table full, out of memory, stream under graph capture): the product
-// then runs without splitting.
-float *split_workspace(hipStream_t stream) {
-    int device;
-    if (hipGetDevice(&device) != hipSuccess) return nullptr;
-    std::lock_guard<std::mutex> lock(workspace_mutex);
-    for (int i = 0; i < num_workspaces; ++i)
-        if (workspaces[i].device == device && workspaces[i].stream == stream) return workspaces[i].pointer;
-    if (num_workspaces == kMaxWorkspaces) return nullptr;
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
-        (void)hipGetLastError();
-        return nullptr;
-    }
-    void *pointer = nullptr;
-    if (hipMalloc(&pointer, sizeof(float) * kPartialFloats * kMaxPartials) != hipSuccess) {
-        (void)hipGetLastError();
-        return nullptr;
-    }
-    workspaces[num_workspaces++] = {device, stream, static_cast<float *>(pointer)};
-    return static_cast<float *>(pointer);
-}
-}  // namespace
-
 // The fused epilogues exist for one layout: both operands K-contiguous, output-sparse mode, T in and out, whole
 // column tiles (the activation width a multiple of 128 for the forward, of 8 for the backward).
 bool mfma_gemm_fusion_eligible(const GemmArgs &args, int dtype) {
@@ -1185,23 +1136,46 @@ bool mfma_gemm_fusion_eligible(const GemmArgs &args, int dtype) {
     return true;
 }
 
-int mfma_gemm_launch(GemmArgs args, int dtype, hipStream_t stream) {
+// ---- workspace for split reductions --------------------------------------------------------------------
+// Whether a product is one whose last round is split is decided from its dimensions alone (few rounds of long tiles);
+// the caller then brings kMaxPartials tile-sized fp32 slots. Given the dimensions, whether the split happens depends
+// on nothing but the presence of the workspace, which is the caller's choice.
+static void count_tiles(GemmArgs &args) {
     if (args.mode == kInputRowSparse) {
         args.tiles_m = static_cast<int>((args.sparse_size + kTile - 1) / kTile) * args.num_experts;
     } else {
         // Upper bound of sum_e ceil(rows_e / 256); surplus workgroups find no tile and exit.
-        args.tiles_m = static_cast<int>((args.rows + kTile - 1) / kTile + (args.expert_ends ? args.num_experts : 0));
+        args.tiles_m = static_cast<int>((args.rows + kTile - 1) / kTile + (args.num_experts > 1 ? args.num_experts : 0));
     }
     args.tiles_n = static_cast<int>((args.cols + kTile - 1) / kTile);
     if (args.fusion == kFusionGatedForward) args.tiles_n = static_cast<int>(args.half / (kTile / 2));
+}
+
+static bool splits_last_round(const GemmArgs &args) {
+    constexpr int kMaxRoundsToSplit = 16;
+    return args.fusion == kFusionNone && args.mode != kInputRowSparse && args.inner / kBK >= 2 * kMinPieceSlices &&
+           static_cast<int64_t>(args.tiles_m) * args.tiles_n <= kMaxRoundsToSplit * kRound;
+}
+
+size_t mfma_gemm_workspace_size(GemmArgs args) {
+    if (args.rows <= 0 || args.cols <= 0 || args.inner <= 0) return 0;
+    count_tiles(args);
+    return splits_last_round(args) ? sizeof(float) * kPartialFloats * kMaxPartials : 0;
+}
+
+int mfma_gemm_launch(GemmArgs args, int dtype, void *workspace, size_t workspace_size, hipStream_t stream) {
+    count_tiles(args);
     if (static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31) - 1024)
         return fail(FM_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
-    // Splitting the last round's reductions can pay when the rounds are few and the reduction is long.
     args.partials = nullptr;
-    constexpr int kMaxRoundsToSplit = 16;
-    if (args.fusion == kFusionNone && args.mode != kInputRowSparse && args.inner / kBK >= 2 * kMinPieceSlices &&
-        static_cast<int64_t>(args.tiles_m) * args.tiles_n <= kMaxRoundsToSplit * kRound && split_enabled())
-        args.partials = split_workspace(stream);
+    if (workspace != nullptr && splits_last_round(args)) {
+        const size_t needed = sizeof(float) * kPartialFloats * kMaxPartials;
+        if (workspace_size < needed || !aligned16(workspace))
+            return fail(FM_ERR_INVALID_ARGUMENT,
+                        "grouped gemm: workspace of %zu bytes (16-byte aligned) needed, got %zu at %p", needed,
+                        workspace_size, workspace);
+        args.partials = static_cast<float *>(workspace);
+    }
     return dtype == FM_DTYPE_BF16 ? launch_layout<bf16_t>(args, stream) : launch_layout<f16_t>(args, stream);
 }
 

@@ -8,6 +8,7 @@ strides, so transposed views (`weight.t()`, `activations.t()`) are consumed in p
 import torch
 
 from fast_llm_amd import _lib
+from fast_llm_amd.functional.config import KernelConfig
 from fast_llm_amd.functional.sparse_copy import SparseMap
 from fast_llm_amd.functional.utils import Assert, div
 
@@ -42,6 +43,14 @@ def _launch(
     pointers = [_lib.ptr(lhs.detach()), _lib.ptr(rhs.detach()), _lib.ptr(out), _lib.ptr(expert_ends)]
     if with_pad_begins:
         pointers.append(_lib.ptr(expert_pad_begins))
+    # Scratch for splitting the last round of a launch with few, long tiles. A torch allocation per call: the caching
+    # allocator hands the same block back to calls on one stream and keeps calls on different streams apart, also
+    # under graph capture. Whether a product splits depends on its dimensions and this switch only.
+    workspace, workspace_size = None, 0
+    if KernelConfig.split_last_round and not with_pad_begins:
+        workspace_size = _lib.lib().fm_grouped_gemm_workspace_size(*dims, num_experts, _lib.dtype_tag(lhs.dtype))
+        if workspace_size:
+            workspace = torch.empty(workspace_size, dtype=torch.uint8, device=device)
     _lib.call(
         name,
         device,
@@ -58,6 +67,8 @@ def _launch(
         _lib.dtype_tag(lhs.dtype),
         _lib.dtype_tag(out.dtype),
         _lib.index_tag(index_dtype),
+        _lib.ptr(workspace),
+        workspace_size,
         label=f"{name}[{dims[0]}x{dims[1]}x{dims[2]}]",
     )
     return out

@@ -4,12 +4,9 @@
  * Every entry point
  *   - takes plain device pointers, 64-bit sizes/strides (in elements) and small integer enums;
  *   - launches asynchronously on the HIP stream passed last (`void *` holding a `hipStream_t`, NULL = default
- *     stream) and never synchronises, frees device memory, or keeps a caller's pointer after it returns. It does
- *     not allocate either, with one exception: the three grouped products keep a workspace of 128 MiB per
- *     (device, stream) for splitting the reductions of a launch's last tiles over idle CUs; it is allocated at a
- *     stream's first product with few tiles and a long reduction (never while the stream is being captured: the
- *     product then runs unsplit) and kept until the process ends. FASTMOE_SPLIT_REDUCTION=0 in the environment
- *     turns the split, and with it the allocation, off;
+ *     stream) and never synchronises, allocates or frees device memory, or keeps a caller's pointer after it
+ *     returns: outputs and every workspace are the caller's, and a workspace may be reused as soon as the stream
+ *     has passed the call;
  *   - returns `FM_OK` (0) or a negative `fm_status`; the message for the calling thread is read with
  *     `fm_last_error()`. No C++ exception crosses this boundary.
  *
@@ -27,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 4
+#define FM_VERSION 5
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -202,8 +199,23 @@ int fm_mlp_activation_backward(const void *grad_output, void *grad_input, const 
  * fast_llm/functional/config.py:106, sparse_linear.py:274). If `expert_ends` is NULL the product is an
  * ordinary dense one (a single expert owning all rows), which is what the reference does for
  * `sparse_map=None` (sparse_linear.py:276-277, 404-405, 537-538).
- * Results are deterministic (no split-K, no floating-point atomics).
+ * Results are deterministic (no floating-point atomics; every sum has a fixed order that depends only on the
+ * arguments and the expert map).
+ *
+ * `workspace`: a launch of few, long tiles (at most 16 rounds of 256 tiles of 256 x 256, reduction of 2048 or more)
+ * leaves most CUs idle in its last round; given `fm_grouped_gemm_workspace_size(...)` bytes of device scratch
+ * (16-byte aligned, content irrelevant) the output-sparse and input-inner-sparse products cut the reductions of that
+ * round's tiles into 2, 4 or 8 pieces that fill the CUs and add the pieces in piece order. Whether this happens
+ * depends on the dimensions and on whether a workspace is passed, on nothing else (not on the stream, the device's
+ * free memory or earlier calls): NULL with size 0 selects the unsplit sums, which differ from the split ones in
+ * the last bits; a non-null workspace smaller than required is FM_ERR_INVALID_ARGUMENT. Calls that may overlap
+ * (different streams) need different workspaces. The row-sparse product never splits and ignores the pair.
  * --------------------------------------------------------------------------------------------------------- */
+
+/* Bytes of workspace with which a product `out [row_dim, col_dim] = lhs [row_dim, inner_dim] x rhs` of `dtype`
+ * operands over `num_experts` experts (1 for a dense product) splits its last round; 0 if it never splits. */
+size_t fm_grouped_gemm_workspace_size(int64_t row_dim, int64_t col_dim, int64_t inner_dim, int64_t num_experts,
+                                      int dtype);
 
 /* out[i, j] = sum_k lhs[i, k] * rhs[k, j + col_sparse_dim * e(i)]   for i < expert_ends[-1]; rows past the last
  * expert ("phantom" rows) are neither read nor written. Padding rows inside an expert are computed like
@@ -213,7 +225,8 @@ int fm_output_sparse_matmul(const void *lhs, const void *rhs, void *out, const v
                             int64_t row_dim, int64_t col_sparse_dim, int64_t inner_dim, int64_t num_experts,
                             int64_t lhs_stride_row, int64_t lhs_stride_inner, int64_t rhs_stride_inner,
                             int64_t rhs_stride_col, int64_t out_stride_row, int64_t out_stride_col,
-                            int accumulate, int dtype, int out_dtype, int index_dtype, void *stream);
+                            int accumulate, int dtype, int out_dtype, int index_dtype, void *workspace,
+                            size_t workspace_size, void *stream);
 
 /* out[i, j] = sum_k lhs[i, k] * rhs[k + inner_sparse_dim * e(i), j]; same row rules as above.
  * lhs [row_dim, inner_sparse_dim], rhs [inner_sparse_dim * num_experts, col_dim], out [row_dim, col_dim].
@@ -222,7 +235,8 @@ int fm_input_inner_sparse_matmul(const void *lhs, const void *rhs, void *out, co
                                  int64_t row_dim, int64_t col_dim, int64_t inner_sparse_dim, int64_t num_experts,
                                  int64_t lhs_stride_row, int64_t lhs_stride_inner, int64_t rhs_stride_inner,
                                  int64_t rhs_stride_col, int64_t out_stride_row, int64_t out_stride_col,
-                                 int accumulate, int dtype, int out_dtype, int index_dtype, void *stream);
+                                 int accumulate, int dtype, int out_dtype, int index_dtype, void *workspace,
+                                 size_t workspace_size, void *stream);
 
 /* out[i + row_sparse_dim * e, j] = sum_{k in [begin_e, expert_pad_begins[e])} lhs[i, k] * rhs[k, j],
  * begin_e = expert_ends[e - 1] (0 for e = 0). Rows of the inner dimension outside that range (padding and
@@ -235,7 +249,7 @@ int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void *out, cons
                                int64_t inner_dim, int64_t num_experts, int64_t lhs_stride_row,
                                int64_t lhs_stride_inner, int64_t rhs_stride_inner, int64_t rhs_stride_col,
                                int64_t out_stride_row, int64_t out_stride_col, int accumulate, int dtype,
-                               int out_dtype, int index_dtype, void *stream);
+                               int out_dtype, int index_dtype, void *workspace, size_t workspace_size, void *stream);
 
 /* Layer 1 of a gated MLP with the activation fused into the product's epilogue: what the reference does with
  * `output_sparse_matmul` (fast_llm/functional/triton/sparse_linear.py:261-306) followed by

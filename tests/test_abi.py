@@ -58,8 +58,21 @@ def test_argument_validation_returns_status_and_message(library):
         _lib.check(status)
     status = library.fm_mlp_activation_forward(None, None, 4, 4, 1, 99, 1, None)
     assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"activation" in library.fm_last_error()
-    status = library.fm_output_sparse_matmul(None, None, None, None, 128, 128, 64, 1, 64, 1, 1, 64, 128, 1, 0, 7, 0, 1, None)
+    status = library.fm_output_sparse_matmul(None, None, None, None, 128, 128, 64, 1, 64, 1, 1, 64, 128, 1, 0, 7, 0, 1, None, 0, None)
     assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"dtype" in library.fm_last_error()
+    status = library.fm_output_sparse_matmul(None, None, None, None, 128, 128, 64, 1, 64, 1, 1, 64, 128, 1, 0, 1, 1, 1, None, 64, None)
+    assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"workspace" in library.fm_last_error()
+
+
+def test_grouped_gemm_workspace_size_depends_on_the_dimensions_only(library):
+    # Layer 2 forward at the Mixtral shape: 66 + 8 row tiles x 16 column tiles, reduction 14336 -> splits.
+    size = library.fm_grouped_gemm_workspace_size(17408, 4096, 14336, 8, 1)
+    assert size == 512 * 256 * 256 * 4
+    assert library.fm_grouped_gemm_workspace_size(17408, 4096, 14336, 8, 2) == size
+    assert library.fm_grouped_gemm_workspace_size(17408, 4096, 14336, 8, 0) == 0  # fp32: generic kernel
+    assert library.fm_grouped_gemm_workspace_size(17408, 28672, 4096, 8, 1) == 0  # layer 1 forward: 29 rounds
+    assert library.fm_grouped_gemm_workspace_size(17408, 4096, 1984, 8, 1) == 0  # short reduction
+    assert library.fm_grouped_gemm_workspace_size(0, 4096, 14336, 8, 1) == 0
 
 
 def test_router_and_fused_entry_points_validate_before_launching(library):

@@ -278,8 +278,8 @@ def test_fused_activation_epilogues_are_bit_identical(activation, recompute_leve
 def test_step_replays_from_a_hip_graph(device):
     """Forward + backward of the block (sparse map included) captured once in a HIP graph and replayed with new
     inputs: every replay, with eager work and synchronisations in between, equals the eager result bit for bit.
-    The warm-up runs on the capture stream, which also gives that stream its split-reduction workspace (the library
-    does not allocate while a stream is being captured)."""
+    The warm-up on the capture stream is what torch asks for before any capture; the library itself needs none (its
+    split-reduction workspace is a torch allocation made inside the captured region)."""
     torch.manual_seed(5)
     tokens, hidden, ffn, experts, k = 512, 256, 2048, 4, 2  # few tiles, long reduction: the split path is taken
     layer = DroplessMoEMLP(hidden, ffn, experts, k, dtype=torch.bfloat16, device=device)

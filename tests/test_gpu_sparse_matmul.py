@@ -346,6 +346,70 @@ def test_split_reduction_of_last_round(experts, inner, other, dtype, device):
     assert max_rel_err(dense_matmul(x_gpu, weight[:inner].to(device)).cpu(), expected) <= tolerance
 
 
+def test_split_does_not_depend_on_stream_or_history(device, library):
+    """Whether the last round is split follows from the dimensions and the caller's choice of a workspace only: the
+    same product on the default stream, on twenty fresh streams and captured into a graph on yet another stream that
+    never ran it gives the same bits; without a workspace it gives the (reproducible) unsplit bits; a workspace that
+    is too small is an error, never a silent change of plan."""
+    from fast_llm_amd import _lib
+    from fast_llm_amd.functional.config import KernelConfig
+
+    experts, inner, other, dtype = 9, 4160, 320, torch.bfloat16
+    case = _ragged_case(experts + inner, experts)
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device, torch.int32)
+    rows = oracle_map.num_rows
+    generator = torch.Generator().manual_seed(21)
+    x, weight = _normal(rows, inner, dtype, generator).to(device), _normal(experts * other, inner, dtype, generator).to(device)
+    assert library.fm_grouped_gemm_workspace_size(rows, other, inner, experts, _lib.dtype_tag(dtype)) > 0
+    assert library.fm_grouped_gemm_workspace_size(rows, other, inner, experts, _lib.dtype_tag(torch.float32)) == 0
+    assert library.fm_grouped_gemm_workspace_size(rows, other, 1024, experts, _lib.dtype_tag(dtype)) == 0
+
+    def product():
+        return output_sparse_matmul(x, weight.t(), sparse_map)
+
+    expected = product()
+    torch.cuda.synchronize()
+    for _ in range(20):
+        stream = torch.cuda.Stream(device=device)
+        stream.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(stream):
+            out = product()
+        stream.synchronize()
+        assert torch.equal(out, expected)
+
+    stream = torch.cuda.Stream(device=device)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        captured = product()
+    for _ in range(3):
+        captured.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, expected)
+        assert torch.equal(product(), expected)  # eager work between the replays
+
+    KernelConfig.split_last_round = False
+    try:
+        unsplit = product()
+        assert torch.equal(product(), unsplit)
+    finally:
+        KernelConfig.split_last_round = True
+    assert not torch.equal(unsplit, expected)  # another order of the same sums
+    assert max_rel_err(unsplit.cpu(), expected.cpu()) <= _MAX_REL[dtype]
+
+    # Straight through the C ABI: a workspace one byte short.
+    size = library.fm_grouped_gemm_workspace_size(rows, other, inner, experts, _lib.dtype_tag(dtype))
+    small = torch.empty(size - 1, dtype=torch.uint8, device=device)
+    out = torch.empty_like(expected)
+    status = library.fm_output_sparse_matmul(
+        x.data_ptr(), weight.data_ptr(), out.data_ptr(), sparse_map.expert_ends.data_ptr(), rows, other, inner, experts,
+        x.stride(0), x.stride(1), 1, inner, other, 1, 0, _lib.dtype_tag(dtype), _lib.dtype_tag(dtype),
+        _lib.index_tag(torch.int32), small.data_ptr(), size - 1, torch.cuda.current_stream(device).cuda_stream,
+    )  # fmt: skip
+    assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"workspace" in library.fm_last_error()
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_random_shapes_through_the_matrix_core_kernel(seed, device):
     """A sweep over ragged expert layouts and sizes around the kernel's tile (256 x 256 x 64), slice-pair and
