@@ -157,28 +157,14 @@ extern "C" size_t fm_sparse_map_workspace_size(int64_t num_rows_dense, int64_t n
     return (bytes + 255) / 256 * 256 + 256;
 }
 
-extern "C" int fm_sparse_map(const int64_t *top_experts, int64_t num_rows_dense, int64_t num_experts_per_token,
-                             int64_t num_experts, int64_t pad_to_multiple, int index_dtype, void *sparse_rows,
-                             void *expert_ends, void *expert_pad_begins, void *workspace, size_t workspace_size,
-                             void *stream_) {
-    using namespace fm;
-    FM_REQUIRE(num_rows_dense >= 0 && num_experts_per_token >= 0, "fm_sparse_map: negative shape");
-    FM_REQUIRE(num_experts >= 1 && num_experts <= kMapMaxExperts,
-               "fm_sparse_map: num_experts=%lld outside [1, %d]", (long long)num_experts, kMapMaxExperts);
-    FM_REQUIRE(pad_to_multiple >= 1, "fm_sparse_map: pad_to_multiple=%lld < 1", (long long)pad_to_multiple);
-    FM_REQUIRE(valid_index_dtype(index_dtype), "fm_sparse_map: bad index_dtype %d", index_dtype);
-    const int64_t num_entries = num_rows_dense * num_experts_per_token;
-    const int64_t max_rows = num_entries + num_experts * pad_to_multiple;
-    FM_REQUIRE(max_rows < (int64_t(1) << 31), "fm_sparse_map: %lld padded rows overflow int32", (long long)max_rows);
-    FM_REQUIRE(index_dtype != FM_INDEX_I16 || max_rows <= 32767 + pad_to_multiple,
-               "fm_sparse_map: %lld padded rows do not fit int16", (long long)max_rows);
-    FM_REQUIRE(expert_ends && expert_pad_begins && workspace, "fm_sparse_map: null output or workspace");
-    FM_REQUIRE(num_entries == 0 || (top_experts && sparse_rows), "fm_sparse_map: null top_experts/sparse_rows");
-    FM_REQUIRE(workspace_size >= fm_sparse_map_workspace_size(num_rows_dense, num_experts_per_token, num_experts),
-               "fm_sparse_map: workspace of %zu bytes is too small", workspace_size);
-    FM_REQUIRE(aligned16(workspace), "fm_sparse_map: workspace must be 16-byte aligned");
+namespace fm {
 
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
+// Validation and the three launches; `workspace` holds fm_sparse_map_workspace_size(...) bytes.
+static int run_sparse_map(const char *name, const int64_t *top_experts, int64_t num_rows_dense,
+                          int64_t num_experts_per_token, int64_t num_experts, int64_t pad_to_multiple, int index_dtype,
+                          void *sparse_rows, void *expert_ends, void *expert_pad_begins, void *workspace,
+                          hipStream_t stream) {
+    const int64_t num_entries = num_rows_dense * num_experts_per_token;
     const int blocks = static_cast<int>(map_num_blocks(num_entries));
     const int experts = static_cast<int>(num_experts);
     int32_t *block_counts = static_cast<int32_t *>(workspace);
@@ -194,5 +180,43 @@ extern "C" int fm_sparse_map(const int64_t *top_experts, int64_t num_rows_dense,
         sparse_map_rows_kernel<<<blocks, kMapBlock, kMapWaves * experts * sizeof(int32_t), stream>>>(
             top_experts, num_entries, experts, block_counts, expert_begins, index_dtype, sparse_rows);
     }
-    return check_launch("fm_sparse_map");
+    return check_launch(name);
+}
+
+static int check_sparse_map_arguments(const char *name, const int64_t *top_experts, int64_t num_rows_dense,
+                                      int64_t num_experts_per_token, int64_t num_experts, int64_t pad_to_multiple,
+                                      int index_dtype, void *sparse_rows, void *expert_ends, void *expert_pad_begins) {
+    FM_REQUIRE(num_rows_dense >= 0 && num_experts_per_token >= 0, "%s: negative shape", name);
+    FM_REQUIRE(num_experts >= 1 && num_experts <= kMapMaxExperts, "%s: num_experts=%lld outside [1, %d]", name,
+               (long long)num_experts, kMapMaxExperts);
+    FM_REQUIRE(pad_to_multiple >= 1, "%s: pad_to_multiple=%lld < 1", name, (long long)pad_to_multiple);
+    FM_REQUIRE(valid_index_dtype(index_dtype), "%s: bad index_dtype %d", name, index_dtype);
+    const int64_t num_entries = num_rows_dense * num_experts_per_token;
+    const int64_t max_rows = num_entries + num_experts * pad_to_multiple;
+    FM_REQUIRE(max_rows < (int64_t(1) << 31), "%s: %lld padded rows overflow int32", name, (long long)max_rows);
+    FM_REQUIRE(index_dtype != FM_INDEX_I16 || max_rows <= 32767 + pad_to_multiple,
+               "%s: %lld padded rows do not fit int16", name, (long long)max_rows);
+    FM_REQUIRE(expert_ends && expert_pad_begins, "%s: null output", name);
+    FM_REQUIRE(num_entries == 0 || (top_experts && sparse_rows), "%s: null top_experts/sparse_rows", name);
+    return FM_OK;
+}
+
+}  // namespace fm
+
+extern "C" int fm_sparse_map(const int64_t *top_experts, int64_t num_rows_dense, int64_t num_experts_per_token,
+                             int64_t num_experts, int64_t pad_to_multiple, int index_dtype, void *sparse_rows,
+                             void *expert_ends, void *expert_pad_begins, void *workspace, size_t workspace_size,
+                             void *stream) {
+    using namespace fm;
+    if (int status = check_sparse_map_arguments("fm_sparse_map", top_experts, num_rows_dense, num_experts_per_token,
+                                                num_experts, pad_to_multiple, index_dtype, sparse_rows, expert_ends,
+                                                expert_pad_begins))
+        return status;
+    FM_REQUIRE(workspace, "fm_sparse_map: null workspace");
+    FM_REQUIRE(workspace_size >= fm_sparse_map_workspace_size(num_rows_dense, num_experts_per_token, num_experts),
+               "fm_sparse_map: workspace of %zu bytes is too small", workspace_size);
+    FM_REQUIRE(aligned16(workspace), "fm_sparse_map: workspace must be 16-byte aligned");
+    return run_sparse_map("fm_sparse_map", top_experts, num_rows_dense, num_experts_per_token, num_experts,
+                          pad_to_multiple, index_dtype, sparse_rows, expert_ends, expert_pad_begins, workspace,
+                          static_cast<hipStream_t>(stream));
 }
