@@ -12,7 +12,7 @@ import torch
 
 LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "csrc" / "libfastmoe_hip.so"
 
-FM_VERSION = 5
+FM_VERSION = 6
 
 _c_i64, _c_int, _c_ptr, _c_size = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
@@ -23,6 +23,8 @@ SIGNATURES: dict[str, tuple] = {
     "fm_last_error": (ctypes.c_char_p, []),
     "fm_sparse_map_workspace_size": (_c_size, [_c_i64] * 3),
     "fm_sparse_map": (_c_int, [_c_ptr] + [_c_i64] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_size, _c_ptr]),
+    "fm_sparse_map_static_scratch_size": (_c_size, []),
+    "fm_sparse_map_static": (_c_int, [_c_ptr] + [_c_i64] * 4 + [_c_int] + [_c_ptr] * 3 + [_c_ptr]),
     "fm_copy_dense_to_sparse": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int] * 3 + [_c_ptr]),
     "fm_copy_sparse_to_dense": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int] * 3 + [_c_ptr]),
     "fm_copy_sparse_to_dense_grad_score": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int] * 3 + [_c_ptr]),

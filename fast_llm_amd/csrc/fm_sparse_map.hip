@@ -15,6 +15,8 @@
 // (reference: fast_llm/functional/triton/sparse_copy.py:249-254).
 #include "fm_common.h"
 
+#include <mutex>
+
 namespace fm {
 
 constexpr int kMapBlock = 1024;  // entries (= threads) per workgroup
@@ -217,6 +219,65 @@ extern "C" int fm_sparse_map(const int64_t *top_experts, int64_t num_rows_dense,
                "fm_sparse_map: workspace of %zu bytes is too small", workspace_size);
     FM_REQUIRE(aligned16(workspace), "fm_sparse_map: workspace must be 16-byte aligned");
     return run_sparse_map("fm_sparse_map", top_experts, num_rows_dense, num_experts_per_token, num_experts,
+                          pad_to_multiple, index_dtype, sparse_rows, expert_ends, expert_pad_begins, workspace,
+                          static_cast<hipStream_t>(stream));
+}
+
+// ---- the same map without any allocation ----------------------------------------------------------------
+// The per-workgroup counts live in a fixed array in device memory that is part of the loaded code object: every GPU
+// the library runs on holds its own copy, at its own address, until the process ends.
+namespace fm {
+
+constexpr size_t kStaticScratchBytes = FM_SPARSE_MAP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+
+// Device address of this device's copy of `scratch`, looked up once per device with that device current. In host
+// code the array's name is not a device address; only the pointer returned here may go to kernels.
+static int static_scratch_of_current_device(void **pointer) {
+    static std::mutex mutex;
+    static void *addresses[kMaxDevices] = {};
+    int device = -1;
+    hipError_t error = hipGetDevice(&device);
+    if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "fm_sparse_map_static: hipGetDevice: %s", hipGetErrorString(error));
+    if (device < 0 || device >= kMaxDevices)
+        return fail(FM_ERR_UNSUPPORTED, "fm_sparse_map_static: device %d outside [0, %d)", device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(mutex);
+    if (addresses[device] == nullptr) {
+        void *address = nullptr;
+        error = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        if (error != hipSuccess || address == nullptr)
+            return fail(FM_ERR_LAUNCH, "fm_sparse_map_static: hipGetSymbolAddress: %s", hipGetErrorString(error));
+        addresses[device] = address;
+    }
+    *pointer = addresses[device];
+    return FM_OK;
+}
+
+}  // namespace fm
+
+extern "C" size_t fm_sparse_map_static_scratch_size(void) { return fm::kStaticScratchBytes; }
+
+extern "C" int fm_sparse_map_static(const int64_t *top_experts, int64_t num_rows_dense, int64_t num_experts_per_token,
+                                    int64_t num_experts, int64_t pad_to_multiple, int index_dtype, void *sparse_rows,
+                                    void *expert_ends, void *expert_pad_begins, void *stream) {
+    using namespace fm;
+    if (int status = check_sparse_map_arguments("fm_sparse_map_static", top_experts, num_rows_dense,
+                                                num_experts_per_token, num_experts, pad_to_multiple, index_dtype,
+                                                sparse_rows, expert_ends, expert_pad_begins))
+        return status;
+    const size_t needed = fm_sparse_map_workspace_size(num_rows_dense, num_experts_per_token, num_experts);
+    if (needed > kStaticScratchBytes)
+        return fail(FM_ERR_UNSUPPORTED,
+                    "fm_sparse_map_static: %lld x %lld entries over %lld experts need %zu bytes of scratch, the fixed "
+                    "array holds %zu; use fm_sparse_map with a workspace",
+                    (long long)num_rows_dense, (long long)num_experts_per_token, (long long)num_experts, needed,
+                    kStaticScratchBytes);
+    void *workspace = nullptr;
+    if (int status = static_scratch_of_current_device(&workspace)) return status;
+    // Nothing to clear: the histogram kernel writes every count the other two kernels read.
+    return run_sparse_map("fm_sparse_map_static", top_experts, num_rows_dense, num_experts_per_token, num_experts,
                           pad_to_multiple, index_dtype, sparse_rows, expert_ends, expert_pad_begins, workspace,
                           static_cast<hipStream_t>(stream));
 }

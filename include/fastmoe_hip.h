@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 5
+#define FM_VERSION 6
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -87,6 +87,21 @@ int fm_sparse_map(const int64_t *top_experts,   /* [num_rows_dense, num_experts_
                   void *expert_ends,            /* [num_experts] */
                   void *expert_pad_begins,      /* [num_experts] */
                   void *workspace, size_t workspace_size, void *stream);
+
+/* The same map for callers that cannot allocate device memory or bring a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid allocation). It has no counterpart in the reference. Same arguments,
+ * results and kernels as `fm_sparse_map`, but the scratch is a fixed array of FM_SPARSE_MAP_STATIC_SCRATCH_BYTES of
+ * device memory inside the library (every GPU the library runs on holds its copy until the process ends), and the
+ * call allocates and frees nothing. Inputs whose `fm_sparse_map_workspace_size(...)` exceeds the array are refused
+ * with FM_ERR_UNSUPPORTED (1 MiB covers e.g. 131072 x 8 entries over 128 experts, or 16384 x 8 over 1024). All calls
+ * on one GPU share that GPU's array: calls that may overlap (different streams, different threads) race; calls on one
+ * stream are safe. The array's address is looked up at a device's first call (a host-side query, no allocation); make
+ * that first call outside graph capture. */
+#define FM_SPARSE_MAP_STATIC_SCRATCH_BYTES (1 << 20)
+size_t fm_sparse_map_static_scratch_size(void);
+int fm_sparse_map_static(const int64_t *top_experts, int64_t num_rows_dense, int64_t num_experts_per_token,
+                         int64_t num_experts, int64_t pad_to_multiple, int index_dtype, void *sparse_rows,
+                         void *expert_ends, void *expert_pad_begins, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------------
  * Sparse copies. `scores` may be NULL (un-scored copy); otherwise [num_rows_dense, num_experts_per_token]
