@@ -37,10 +37,22 @@ def _activation_tag(activation_type: ActivationType | str) -> int:
     return _lib.ACTIVATIONS[name]
 
 
-def mlp_activation_forward(input_: torch.Tensor, gated: bool, activation_type: ActivationType):
+def _row_limit(sparse_map: SparseMap | None, tensor: torch.Tensor) -> tuple[int | None, int]:
+    """(device address of the number of rows in use, its index tag) for a [num_rows, ...] buffer of `sparse_map`: the
+    last entry of `expert_ends`. The rows after it belong to no expert and need not be streamed through."""
+    if sparse_map is None or tensor.dim() != 2 or tensor.size(0) != sparse_map.num_rows:
+        return None, 0
+    ends = sparse_map.expert_ends
+    return ends.data_ptr() + (ends.numel() - 1) * ends.element_size(), _lib.index_tag(ends.dtype)
+
+
+def mlp_activation_forward(
+    input_: torch.Tensor, gated: bool, activation_type: ActivationType, sparse_map: SparseMap | None = None
+):
     """
     out = act(input_[..., :n]) * input_[..., n:] if gated else act(input_).
-    Reference: `triton_mlp_activation_forward`, fast_llm/functional/triton/mlp.py:142-162.
+    Reference: `triton_mlp_activation_forward`, fast_llm/functional/triton/mlp.py:142-162. With `sparse_map` (not in
+    the reference's signature) the rows past the last expert's end are skipped instead of computed from garbage.
     """
     assert input_.is_contiguous()
     device = _lib.require_device(input_)
@@ -56,8 +68,9 @@ def mlp_activation_forward(input_: torch.Tensor, gated: bool, activation_type: A
         int(gated),
         _activation_tag(activation_type),
         _lib.dtype_tag(input_.dtype),
+        *_row_limit(sparse_map, input_),
     )
-    return output, (input_, gated, activation_type)
+    return output, (input_, gated, activation_type, sparse_map)
 
 
 def mlp_activation_backward(grad_output: torch.Tensor, context: tuple, recompute: bool = False):
@@ -66,7 +79,8 @@ def mlp_activation_backward(grad_output: torch.Tensor, context: tuple, recompute
     Reference: `triton_mlp_activation_backward`, fast_llm/functional/triton/mlp.py:165-190.
     """
     assert grad_output.is_contiguous()
-    input_, gated, activation_type = context
+    input_, gated, activation_type, *rest = context
+    sparse_map = rest[0] if rest else None
     device = _lib.require_device(input_, grad_output)
     grad_input = torch.empty_like(input_)
     output = torch.empty_like(grad_output) if recompute else None
@@ -83,6 +97,7 @@ def mlp_activation_backward(grad_output: torch.Tensor, context: tuple, recompute
         int(gated),
         _activation_tag(activation_type),
         _lib.dtype_tag(input_.dtype),
+        *_row_limit(sparse_map, input_),
     )
     return grad_input, output
 
@@ -224,7 +239,7 @@ def mlp_forward(
         intermediate_1, _ = output_parallel_linear_forward(
             intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
         )
-        intermediate_2, _ = mlp_activation_forward(intermediate_1, gated, activation_type)
+        intermediate_2, _ = mlp_activation_forward(intermediate_1, gated, activation_type, sparse_map)
 
     if recompute_level.recompute_sparse_input:
         intermediate_0 = None
@@ -336,7 +351,7 @@ def mlp_backward(grad_output: torch.Tensor, context: list[typing.Any]) -> tuple[
         else:
             grad_intermediate_2 = output_sparse_matmul(grad_output, weight_2_t, sparse_map)
         grad_intermediate_1, intermediate_2_ = mlp_activation_backward(
-            grad_intermediate_2.contiguous(), (intermediate_1, gated, activation_type), intermediate_2 is None
+            grad_intermediate_2.contiguous(), (intermediate_1, gated, activation_type, sparse_map), intermediate_2 is None
         )
         del grad_intermediate_2
 

@@ -95,6 +95,7 @@ def _copy_arguments(dense: torch.Tensor, sparse: torch.Tensor, scores: torch.Ten
     Assert.eq(sparse.dim(), 2)
     Assert.eq(dense.size(0), sparse_map.num_rows_dense)
     Assert.eq(dense.size(1), sparse.size(1))
+    Assert.eq(sparse.size(0), sparse_map.num_rows)
     Assert.eq(dense.dtype, sparse.dtype)
     Assert.eq(tuple(sparse_map.sparse_rows.shape), (sparse_map.num_rows_dense, sparse_map.num_experts_per_token))
     assert dense.is_contiguous() and sparse.is_contiguous() and sparse_map.sparse_rows.is_contiguous()

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 6
+#define FM_VERSION 7
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -106,7 +106,8 @@ int fm_sparse_map_static(const int64_t *top_experts, int64_t num_rows_dense, int
 /* ---------------------------------------------------------------------------------------------------------
  * Sparse copies. `scores` may be NULL (un-scored copy); otherwise [num_rows_dense, num_experts_per_token]
  * of `scores_dtype`. All row-major contiguous with `num_columns` columns. `num_rows_sparse` is the row
- * count of the sparse buffer and is only used to bound-check nothing on the device; it documents the shape.
+ * count of the sparse buffer: entries of `sparse_rows` outside [0, num_rows_sparse) are skipped (not copied, and
+ * they add nothing to a combine or a score gradient, which is 0 for them), never dereferenced.
  * --------------------------------------------------------------------------------------------------------- */
 
 /* Dispatch: output[sparse_rows[t, j], :] = input[t, :] * (scores[t, j] or 1), product in fp32, one rounding.
@@ -193,17 +194,21 @@ int fm_router_backward(const void *grad_scores, const void *scores, const void *
 /* ---------------------------------------------------------------------------------------------------------
  * MLP activation. `input` is [num_rows, num_columns * (gated ? 2 : 1)], `output`/`grad_output` are
  * [num_rows, num_columns]; all contiguous. Gated: out = act(in[:, :n]) * in[:, n:]. Math in fp32.
+ * `row_limit` (may be NULL) points to one device integer of `index_dtype`, the number of rows in use: rows at and
+ * past it are neither read nor written. Passing the address of the last entry of a sparse map's `expert_ends`
+ * keeps the kernels off the rows of the static worst-case layout that no expert owns (the reference's kernels
+ * stream through them; nothing ever reads what they produce there).
  * --------------------------------------------------------------------------------------------------------- */
 
 /* Replaces `triton_mlp_activation_forward_kernel` (fast_llm/functional/triton/mlp.py:29-71, launched :153-162). */
 int fm_mlp_activation_forward(const void *input, void *output, int64_t num_rows, int64_t num_columns, int gated,
-                              int activation, int dtype, void *stream);
+                              int activation, int dtype, const void *row_limit, int index_dtype, void *stream);
 
 /* grad_input has the shape of input. `output` (may be NULL) receives the recomputed forward output.
  * Replaces `triton_mlp_activation_backward_kernel` (mlp.py:74-139, launched :177-189). */
 int fm_mlp_activation_backward(const void *grad_output, void *grad_input, const void *input, void *output,
                                int64_t num_rows, int64_t num_columns, int gated, int activation, int dtype,
-                               void *stream);
+                               const void *row_limit, int index_dtype, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------------
  * Grouped ("sparse") matrix products. Strides are in elements. `lhs`/`rhs` share `dtype`; `out` has

@@ -56,7 +56,7 @@ def test_argument_validation_returns_status_and_message(library):
     assert b"num_experts" in library.fm_last_error()
     with pytest.raises(ValueError, match="num_experts"):
         _lib.check(status)
-    status = library.fm_mlp_activation_forward(None, None, 4, 4, 1, 99, 1, None)
+    status = library.fm_mlp_activation_forward(None, None, 4, 4, 1, 99, 1, None, 0, None)
     assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"activation" in library.fm_last_error()
     status = library.fm_output_sparse_matmul(None, None, None, None, 128, 128, 64, 1, 64, 1, 1, 64, 128, 1, 0, 7, 0, 1, None, 0, None)
     assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"dtype" in library.fm_last_error()

@@ -73,3 +73,39 @@ def test_silu_extremes_are_finite(device):
 def test_sigmoid_has_no_kernel(device):
     with pytest.raises(NotImplementedError):
         mlp_activation_forward(torch.zeros(2, 4, device=device), False, ActivationType.sigmoid)
+
+
+@pytest.mark.parametrize("index_dtype", [torch.int16, torch.int32, torch.int64])
+@pytest.mark.parametrize("limit", [0, 1, 37, 64, 200])
+def test_rows_past_the_limit_are_left_alone(limit, index_dtype, device, library):
+    """With a device-side row limit (the last entry of a sparse map's `expert_ends`) the kernels neither read nor write
+    the rows after it: outputs keep their sentinel there, rows before it equal the unlimited result, and NaN stored in
+    the skipped input rows changes nothing."""
+    from fast_llm_amd import _lib
+
+    rows, columns = 64, 384
+    generator = torch.Generator().manual_seed(limit)
+    input_ = torch.randn(rows, 2 * columns, generator=generator).to(torch.bfloat16).to(device)
+    grad_output = torch.randn(rows, columns, generator=generator).to(torch.bfloat16).to(device)
+    expected, context = mlp_activation_forward(input_, True, ActivationType.silu)
+    expected_grad, _ = mlp_activation_backward(grad_output, context)
+    used = min(limit, rows)
+    input_[used:] = float("nan")
+    ends = torch.tensor([5, limit], dtype=index_dtype, device=device)
+    limit_pointer = ends.data_ptr() + ends.element_size()
+    stream = torch.cuda.current_stream(device).cuda_stream
+    tags = (1, _lib.ACTIVATIONS["silu"], _lib.dtype_tag(torch.bfloat16), limit_pointer, _lib.index_tag(index_dtype), stream)
+
+    output = torch.full((rows, columns), 3.0, dtype=torch.bfloat16, device=device)
+    _lib.check(library.fm_mlp_activation_forward(input_.data_ptr(), output.data_ptr(), rows, columns, *tags))
+    assert torch.equal(output[:used], expected[:used]) and (output[used:] == 3.0).all()
+
+    grad_input = torch.full((rows, 2 * columns), 3.0, dtype=torch.bfloat16, device=device)
+    recomputed = torch.full((rows, columns), 3.0, dtype=torch.bfloat16, device=device)
+    _lib.check(
+        library.fm_mlp_activation_backward(
+            grad_output.data_ptr(), grad_input.data_ptr(), input_.data_ptr(), recomputed.data_ptr(), rows, columns, *tags
+        )
+    )
+    assert torch.equal(grad_input[:used], expected_grad[:used]) and (grad_input[used:] == 3.0).all()
+    assert torch.equal(recomputed[:used], expected[:used]) and (recomputed[used:] == 3.0).all()

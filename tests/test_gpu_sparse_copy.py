@@ -168,3 +168,61 @@ def test_full_size_round_trip(name, device):
     grad_scores = copy_sparse_to_dense_grad_score(sparse, x, sparse_map)
     expected = (x.float() ** 2).sum(1, keepdim=True).expand(-1, k)  # <x_t, x_t> for every slot
     assert max_rel_err(grad_scores, expected) <= 1e-2
+
+
+def test_rows_outside_the_sparse_buffer_are_skipped(device, library):
+    """Entries of `sparse_rows` that are negative or not below the sparse buffer's row count (a map built for another
+    buffer) are skipped by all four kernels, never dereferenced: such a slot copies nothing, adds nothing to the
+    combine and gets score gradient 0. The Python wrappers refuse a buffer whose row count differs from the map's."""
+    tokens, hidden, k, rows = 40, 256, 3, 128
+    generator = torch.Generator().manual_seed(4)
+    dense = torch.randn(tokens, hidden, generator=generator).to(torch.bfloat16)
+    sparse = torch.randn(rows, hidden, generator=generator).to(torch.bfloat16)
+    scores = torch.rand(tokens, k, generator=generator)
+    sparse_rows = torch.randperm(rows, generator=generator)[: tokens * k].view(tokens, k).to(torch.int32)
+    bad = torch.rand(tokens, k, generator=generator) < 0.3
+    bad_values = torch.where(torch.rand(tokens, k, generator=generator) < 0.5, -1, rows + 1000)
+    bad_rows = torch.where(bad, bad_values, sparse_rows).to(torch.int32)
+    valid = (~bad).float()
+
+    dense_d, sparse_d, scores_d, rows_d = (t.to(device) for t in (dense, sparse, scores, bad_rows))
+    stream = torch.cuda.current_stream(device).cuda_stream
+    shape = (tokens, hidden, k, rows)
+    tags = (_lib.dtype_tag(torch.bfloat16), _lib.dtype_tag(torch.float32), _lib.index_tag(torch.int32), stream)
+
+    out = torch.full((rows, hidden), 7.0, dtype=torch.bfloat16, device=device)
+    _lib.check(library.fm_copy_dense_to_sparse(dense_d.data_ptr(), scores_d.data_ptr(), rows_d.data_ptr(),
+                                               out.data_ptr(), *shape, *tags))  # fmt: skip
+    expected = torch.full((rows, hidden), 7.0, dtype=torch.bfloat16)
+    for t in range(tokens):
+        for j in range(k):
+            if not bad[t, j]:
+                expected[sparse_rows[t, j]] = (dense[t].float() * scores[t, j]).to(torch.bfloat16)
+    assert torch.equal(out.cpu(), expected)
+
+    combined = torch.empty(tokens, hidden, dtype=torch.bfloat16, device=device)
+    _lib.check(library.fm_copy_sparse_to_dense(sparse_d.data_ptr(), scores_d.data_ptr(), rows_d.data_ptr(),
+                                               combined.data_ptr(), *shape, *tags))  # fmt: skip
+    gathered = sparse[sparse_rows.long()].float() * (scores * valid)[:, :, None]
+    assert max_rel_err(combined.cpu(), gathered.sum(1)) <= 1e-2
+
+    grad_scores = torch.empty(tokens, k, dtype=torch.float32, device=device)
+    grad_input = torch.full((rows, hidden), 7.0, dtype=torch.bfloat16, device=device)
+    _lib.check(library.fm_copy_sparse_to_dense_backward(
+        sparse_d.data_ptr(), dense_d.data_ptr(), scores_d.data_ptr(), rows_d.data_ptr(), grad_input.data_ptr(),
+        grad_scores.data_ptr(), *shape, tags[0], tags[1], _lib.dtype_tag(torch.float32), tags[2], stream))  # fmt: skip
+    expected_scores = (sparse[sparse_rows.long()].float() * dense.float()[:, None, :]).sum(-1) * valid
+    assert max_rel_err(grad_scores.cpu(), expected_scores) <= 1e-5
+    assert (grad_scores.cpu()[bad] == 0).all()
+    assert torch.equal(grad_input.cpu(), expected)
+
+    plain = torch.empty(tokens, k, dtype=torch.float32, device=device)
+    _lib.check(library.fm_copy_sparse_to_dense_grad_score(
+        sparse_d.data_ptr(), dense_d.data_ptr(), rows_d.data_ptr(), plain.data_ptr(), *shape, tags[0],
+        _lib.dtype_tag(torch.float32), tags[2], stream))  # fmt: skip
+    assert torch.equal(plain, grad_scores)
+
+    oracle_map, _, _, _ = _problem(tokens, 4, 2, hidden, torch.bfloat16)
+    sparse_map = to_device_map(oracle_map, device, torch.int32)
+    with pytest.raises(AssertionError):
+        copy_sparse_to_dense(torch.zeros(oracle_map.num_rows - 128, hidden, dtype=torch.bfloat16, device=device), None, sparse_map)
