@@ -3,33 +3,41 @@ Benchmark of the dropless-MoE hot path on one MI355X.
 
 A step is one forward + backward of the MoE MLP over one batch of synthetic tokens: sparse map, dispatch, layer 1,
 gated SiLU, layer 2, combine, and the whole backward including both weight gradients. Inputs, weights and routing
-(top-k experts, fp32 scores) are resident in HBM before the timed region. The default workload is the Mixtral-like
+(top-k experts, fp32 scores) are resident in HBM before the timed region. The headline workload is the Mixtral-like
 configuration (8192 tokens, hidden 4096, ffn 14336, 8 experts, top-2, bf16 with fp32 accumulation).
 
 Prints one JSON line: whole-step tokens/s, the roofline of the grouped-GEMM kernel (six launches per step, algorithmic
 FLOPs 18*M*H*F over their summed device time from HIP events on the launch stream), per-kernel figures for the
-bandwidth-bound kernels, and a CPU baseline (the looped torch MoE on the host cores, on a bounded token sample).
+bandwidth-bound kernels, the same step with fp32 gradient buffers, the other four configurations (`configs`), and a
+CPU baseline (the looped torch MoE on the host cores, on a bounded token sample).
+
+`python bench.py --ceilings` prints, instead, what the device sustains: back-to-back MFMAs on zero and on random
+operands, the vendor BLAS on dense products of the same sizes, and a plain streaming copy.
 """
 
 import argparse
 import json
 import os
 import pathlib
+import statistics
 import sys
 import time
 
 import torch
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
+PEAK_FP32_TFLOPS = 157.3  # MI355X fp32 (matrix) peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E peak, GB/s
-# HBM traffic per GEMM launch cannot be measured from inside the process; it comes from the committed summary of two
-# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, WRITE_SIZE, calibrated on the copy kernel below).
-TRAFFIC_SUMMARY = pathlib.Path(__file__).resolve().parent / "profiles" / "bench_mixtral_hbm_traffic.json"
+PROFILES = pathlib.Path(__file__).resolve().parent / "profiles"
+HEADLINE = "mixtral"
+OTHER_WORKLOADS = ("tiny", "fine_grained", "wide", "imbalanced")
 
 
 def measured_traffic(workload_name: str) -> tuple[int | None, str | None]:
+    """HBM traffic per GEMM launch cannot be measured from inside the process; it comes from the committed summary of
+    two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, WRITE_SIZE, calibrated on the add kernel below)."""
     try:
-        summary = json.loads(TRAFFIC_SUMMARY.read_text())
+        summary = json.loads((PROFILES / f"bench_{workload_name}_hbm_traffic.json").read_text())
     except (OSError, ValueError):
         return None, None
     if summary.get("workload") != workload_name:
@@ -40,32 +48,41 @@ def measured_traffic(workload_name: str) -> tuple[int | None, str | None]:
 def parse_args() -> argparse.Namespace:
     parser = argparse.ArgumentParser(description=__doc__)
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=10)
+    parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=3)
-    parser.add_argument("--workload", default="mixtral", help="tiny | mixtral | fine_grained | wide | imbalanced")
+    parser.add_argument("--workload", default=HEADLINE, help="tiny | mixtral | fine_grained | wide | imbalanced")
     parser.add_argument("--recompute", default="none", help="none | activation | activation_and_input | full")
-    parser.add_argument("--cpu-tokens", type=int, default=8192, help="tokens in the CPU baseline sample (0: skip)")
+    parser.add_argument(
+        "--cpu-tokens", type=int, default=4096, help="tokens in the CPU baseline sample of the headline (0: skip)"
+    )
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument(
         "--grad-dtype",
         default="same",
         choices=("same", "fp32"),
-        help="dtype of the weight-gradient buffers: the weights' own (what the reference's kernel benchmarks and "
-        "functional tests attach: torch.empty_like(param)) or float32 (the training engine's full_precision_gradients)",
+        help="dtype of the weight-gradient buffers of the headline: the weights' own (what the reference's kernel "
+        "benchmarks and functional tests attach: torch.empty_like(param)) or float32 (the training engine's "
+        "full_precision_gradients); the other one is reported under `other_grad_dtype`",
     )
+    parser.add_argument(
+        "--only", action="store_true", help="time the chosen workload only (no other configurations, no second "
+        "gradient dtype): what the profiler runs use"
+    )  # fmt: skip
     parser.add_argument(
         "--calibration-mib",
         type=int,
         default=1024,
-        help="size of a plain device copy done once before the warm-up; hardware counters (FETCH_SIZE, WRITE_SIZE) "
+        help="size of a plain device add done once before the warm-up; hardware counters (FETCH_SIZE, WRITE_SIZE) "
         "read for it calibrate the counters read for the kernels of the timed region (0: skip)",
     )
+    parser.add_argument("--ceilings", action="store_true", help="measure the device's ceilings instead of the path")
     return parser.parse_args()
 
 
-def cpu_baseline(workload, inputs, tokens: int) -> dict:
+def cpu_baseline(workload, inputs, tokens: int, repetitions: int = 3) -> dict:
     """The looped torch MoE (per-expert gather -> linear -> silu*up -> linear -> scaled scatter-add, autograd
-    backward) in fp32 on the host cores, over the first `tokens` tokens of the same batch with all experts' weights."""
+    backward) in fp32 on the host cores, over the first `tokens` tokens of the same batch with all experts' weights:
+    one warm-up pass, then the median of `repetitions` timed passes."""
     from oracle import moe_oracle
 
     torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "1024")))))
@@ -80,47 +97,33 @@ def cpu_baseline(workload, inputs, tokens: int) -> dict:
         )
         return time.perf_counter() - start
 
-    run(min(tokens, 32))  # thread pool and allocator warm-up
-    seconds = run(tokens)
+    run(min(tokens, 256))  # thread pool, allocator and page-fault warm-up
+    seconds = [run(tokens) for _ in range(repetitions)]
+    median = statistics.median(seconds)
     return {
-        "value": tokens / seconds,
+        "value": tokens / median,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"first {tokens} of {workload.tokens} tokens, full {workload.experts}-expert weights, fp32, "
-        f"looped torch MoE fwd+bwd, 1 warm-up + 1 timed pass ({seconds:.2f} s)",
+        "sample": f"{workload.name}: first {tokens} of {workload.tokens} tokens, full {workload.experts}-expert weights, "
+        f"fp32, looped torch MoE fwd+bwd, 1 warm-up + {repetitions} timed passes, median "
+        f"({', '.join(f'{s:.2f}' for s in seconds)} s)",
     }
 
 
-def main() -> None:
-    args = parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print(
-            "bench.py measures one GPU: the dropless-MoE path keeps the whole expert set on a single MI355X and has no "
-            "collectives. Run it with --gpus 1.",
-            file=sys.stderr,
-        )
-        sys.exit(2)
-
+def time_workload(workload, args, steps: int, warmup: int, grad_dtype_name: str, recompute_level, device) -> dict:
+    """Warm up, time `steps` steps of `workload` and return the step time and the per-kernel figures."""
     from fast_llm_amd import _lib
-    from fast_llm_amd.functional.config import ActivationType, MLPRecomputeLevel
+    from fast_llm_amd.functional.config import ActivationType
     from fast_llm_amd.functional.mlp import mlp_autograd
     from fast_llm_amd.functional.sparse_copy import get_sparse_map
     from fast_llm_amd.layers.moe import attach_grad_buffer
-    from fast_llm_amd.workloads import WORKLOADS, make_inputs
+    from fast_llm_amd.workloads import make_inputs
 
-    if not _lib.LIBRARY_PATH.is_file():
-        from fast_llm_amd.build import build_library
-
-        build_library()
-
-    workload = WORKLOADS[args.workload]
-    recompute_level = MLPRecomputeLevel(args.recompute)
-    device = torch.device("cuda:0")
     inputs = make_inputs(workload, seed=args.seed, weight_device=device).to(device)
     x = inputs.hidden_states.requires_grad_(True)
     scores = inputs.scores.requires_grad_(True)
-    grad_dtype = torch.float32 if args.grad_dtype == "fp32" else None
+    grad_dtype = torch.float32 if grad_dtype_name == "fp32" else None
     weight_1 = attach_grad_buffer(inputs.weight_1.requires_grad_(True), grad_dtype)
     weight_2 = attach_grad_buffer(inputs.weight_2.requires_grad_(True), grad_dtype)
 
@@ -131,32 +134,27 @@ def main() -> None:
         output = mlp_autograd(
             x, scores, weight_1, None, weight_2, None, True, ActivationType.silu, None, False, True,
             recompute_level, True, sparse_map,
-        )
+        )  # fmt: skip
         output.backward(inputs.grad_output)
 
-    if args.calibration_mib > 0:
-        # One read and one write of a known size, outside the timed region: an elementwise add kernel (a plain
-        # `copy_` would go through the runtime's blit path, for which no counters are reported).
-        source = torch.ones(args.calibration_mib << 18, dtype=torch.float32, device=device)
-        torch.add(source, 1.0, out=torch.empty_like(source))
-        del source
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     with _lib.KernelTimer() as timer:
         start = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             step()
         torch.cuda.synchronize()
         seconds = time.perf_counter() - start
-    ms_per_step = seconds / args.steps * 1e3
-    tokens_per_second = workload.tokens * args.steps / seconds
+    ms_per_step = seconds / steps * 1e3
 
     # Per-kernel device time, averaged over the timed steps.
-    durations = {label: sum(values) / len(values) for label, values in timer.durations_ms().items()}
-    calls_per_step = {label: len(values) / args.steps for label, values in timer.durations_ms().items()}
+    all_durations = timer.durations_ms()
+    durations = {label: sum(values) / len(values) for label, values in all_durations.items()}
+    calls_per_step = {label: len(values) / steps for label, values in all_durations.items()}
     rows, hidden, ffn = workload.sparse_rows_unpadded, workload.hidden, workload.ffn
     itemsize = workload.dtype.itemsize
+    peak_tflops = PEAK_FP32_TFLOPS if workload.dtype == torch.float32 else PEAK_BF16_TFLOPS
     gemm_ms = sum(durations[label] * calls_per_step[label] for label in durations if "matmul" in label)
     gemm_launches = sum(calls_per_step[label] for label in durations if "matmul" in label)
     gemm_flops = workload.gemm_flops * (4 / 3 if recompute_level.recompute_layer_1 else 1)
@@ -171,7 +169,7 @@ def main() -> None:
             # Dimensions are padded/static; algorithmic FLOPs use the unpadded row count.
             per_launch = 2 * rows * (n if "row_sparse" not in label else m) * (k if "row_sparse" not in label else n)
             entry["tflops"] = round(per_launch / (ms * 1e-3) / 1e12, 1)
-            entry["frac_of_mfma_peak"] = round(entry["tflops"] / PEAK_BF16_TFLOPS, 4)
+            entry["frac_of_mfma_peak"] = round(entry["tflops"] / peak_tflops, 4)
         elif label in ("fm_copy_dense_to_sparse", "fm_copy_sparse_to_dense"):
             entry["gbs"] = round(copy_bytes / (ms * 1e-3) / 1e9, 1)
             entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
@@ -184,49 +182,233 @@ def main() -> None:
             entry["gbs"] = round(factor * rows * ffn * itemsize / (ms * 1e-3) / 1e9, 1)
             entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
         kernels[label] = entry
+    return {
+        "inputs": inputs,
+        "ms_per_step": ms_per_step,
+        "tokens_per_s": workload.tokens * steps / seconds,
+        "gemm_ms": gemm_ms,
+        "gemm_launches": gemm_launches,
+        "gemm_flops": gemm_flops,
+        "gemm_tflops": gemm_tflops,
+        "gemm_peak_tflops": peak_tflops,
+        "kernels": kernels,
+    }
 
+
+def summary_of(workload, timed: dict) -> dict:
+    """The per-configuration record: absolute throughput, TFLOP/s and GB/s, and each as a fraction of its roofline."""
+    kernels = timed["kernels"]
+
+    def hbm(label: str) -> dict | None:
+        entry = kernels.get(label)
+        return None if entry is None else {"gbs": entry["gbs"], "frac": entry["frac_of_hbm_peak"]}
+
+    return {
+        "workload": f"{workload.tokens} tokens, hidden {workload.hidden}, ffn {workload.ffn}, {workload.experts} "
+        f"experts, top-{workload.experts_per_token}, {str(workload.dtype).removeprefix('torch.')}",
+        "ms_per_step": round(timed["ms_per_step"], 4),
+        "tokens_per_s": round(timed["tokens_per_s"], 1),
+        "gemm_tflops": round(timed["gemm_tflops"], 1),
+        "gemm_peak_tflops": timed["gemm_peak_tflops"],
+        "gemm_frac": round(timed["gemm_tflops"] / timed["gemm_peak_tflops"], 4),
+        "gemm_frac_of_step": round(timed["gemm_ms"] / timed["ms_per_step"], 4),
+        "dispatch": hbm("fm_copy_dense_to_sparse"),
+        "combine": hbm("fm_copy_sparse_to_dense"),
+        "combine_backward": hbm("fm_copy_sparse_to_dense_backward"),
+        "activation_forward": hbm("fm_mlp_activation_forward"),
+        "activation_backward": hbm("fm_mlp_activation_backward"),
+        "sparse_map_ms": kernels.get("fm_sparse_map", {}).get("ms"),
+    }
+
+
+def release(timed: dict) -> None:
+    timed.pop("inputs", None)
+    torch.cuda.empty_cache()
+
+
+def measure_ceilings(device: torch.device) -> dict:
+    """What the device sustains, for setting the kernels' figures against: see the module docstring."""
+    from fast_llm_amd import _lib
+
+    library = _lib.lib()
+    stream = torch.cuda.current_stream(device)
+    compute_units = torch.cuda.get_device_properties(device).multi_processor_count
+
+    def timed(function, repetitions: int) -> float:
+        function()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(repetitions):
+            function()
+        end.record(stream)
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / repetitions  # ms
+
+    result: dict = {"compute_units": compute_units}
+    sink = torch.empty(compute_units * 256, dtype=torch.float32, device=device)
+    iterations = 40000  # about 30 ms per launch at the published peak
+    flops = library.fm_probe_mfma_flops(compute_units, iterations)
+    for name, random_operands, sigma in (("zeros", 0, 0.0), ("normal_sigma_0.02", 1, 0.02), ("normal_sigma_1", 1, 1.0)):
+        ms = timed(
+            lambda: _lib.check(
+                library.fm_probe_mfma(sink.data_ptr(), compute_units, iterations, random_operands, sigma, stream.cuda_stream)
+            ),
+            10,
+        )
+        result[f"mfma_loop_tflops_{name}"] = round(flops / ms / 1e9, 1)
+
+    # The vendor BLAS (torch.matmul) on dense products of the grouped products' sizes and operand layouts.
+    generator = torch.Generator(device=device).manual_seed(0)
+
+    def normal(*shape):
+        return torch.empty(*shape, dtype=torch.bfloat16, device=device).normal_(0, 0.02, generator=generator)
+
+    rows, hidden, wide = 16384, 4096, 28672
+    x, weight, y = normal(rows, hidden), normal(wide, hidden), normal(rows, wide)
+    gemm_flops = 2 * rows * hidden * wide
+    for name, function in (
+        ("blas_dense_tflops_x_wT", lambda: torch.matmul(x, weight.t())),
+        ("blas_dense_tflops_y_w", lambda: torch.matmul(y, weight)),
+        ("blas_dense_tflops_yT_x", lambda: torch.matmul(y.t(), x)),
+    ):
+        result[name] = round(gemm_flops / timed(function, 10) / 1e9, 1)
+    x_zero, weight_zero = torch.zeros_like(x), torch.zeros_like(weight)
+    result["blas_dense_tflops_x_wT_zeros"] = round(gemm_flops / timed(lambda: torch.matmul(x_zero, weight_zero.t()), 10) / 1e9, 1)
+    del x, weight, y, x_zero, weight_zero
+
+    # Plain copies: 1 GiB read + 1 GiB written.
+    size = 1 << 30
+    source = torch.empty(size, dtype=torch.uint8, device=device).random_(0, 255)
+    target = torch.empty_like(source)
+    for workgroups in (compute_units * 8, compute_units * 32, size // 16 // 256):
+        ms = timed(
+            lambda: _lib.check(
+                library.fm_probe_copy(source.data_ptr(), target.data_ptr(), size, workgroups, stream.cuda_stream)
+            ),
+            20,
+        )
+        result[f"copy_kernel_gbs_{workgroups}_workgroups"] = round(2 * size / ms / 1e6, 1)
+    assert torch.equal(source, target)
+    result["torch_copy_gbs"] = round(2 * size / timed(lambda: target.copy_(source), 20) / 1e6, 1)
+    result["torch_add_gbs"] = round(2 * size / timed(lambda: torch.add(source, 1, out=target), 20) / 1e6, 1)
+    result["peaks"] = {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "hbm_gbs": PEAK_HBM_GBS}
+    return result
+
+
+def main() -> None:
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(
+            "bench.py measures one GPU: the dropless-MoE path keeps the whole expert set on a single MI355X and has no "
+            "collectives. Run it with --gpus 1.",
+            file=sys.stderr,
+        )
+        sys.exit(2)
+
+    from fast_llm_amd import _lib
+    from fast_llm_amd.functional.config import MLPRecomputeLevel
+    from fast_llm_amd.workloads import WORKLOADS
+
+    if not _lib.LIBRARY_PATH.is_file():
+        from fast_llm_amd.build import build_library
+
+        build_library()
+
+    device = torch.device("cuda:0")
+    if args.ceilings:
+        print(json.dumps({"ceilings": measure_ceilings(device)}))
+        return
+
+    workload = WORKLOADS[args.workload]
+    recompute_level = MLPRecomputeLevel(args.recompute)
+    dtype_names = {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}
+
+    if args.calibration_mib > 0:
+        # One read and one write of a known size, outside the timed region: an elementwise add kernel (a plain
+        # `copy_` would go through the runtime's blit path, for which no counters are reported).
+        source = torch.ones(args.calibration_mib << 18, dtype=torch.float32, device=device)
+        torch.add(source, 1.0, out=torch.empty_like(source))
+        del source
+
+    timed = time_workload(workload, args, args.steps, args.warmup, args.grad_dtype, recompute_level, device)
+    hidden, ffn = workload.hidden, workload.ffn
+    grad_dtype_name = "f32" if args.grad_dtype == "fp32" else dtype_names[workload.dtype]
     traffic, traffic_source = measured_traffic(workload.name)
     result = {
         "metric": "MoE fwd+bwd tokens/s at Mixtral shape; grouped-GEMM % bf16 MFMA peak",
-        "value": tokens_per_second,
+        "value": timed["tokens_per_s"],
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": timed["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[workload.dtype],
+        "dtype": dtype_names[workload.dtype],
         "data": "synthetic",
         "config": {
             "workload": f"{workload.name}: dropless MoE MLP fwd+bwd, {workload.tokens} tokens, hidden {hidden}, "
             f"ffn {ffn}, {workload.experts} experts, top-{workload.experts_per_token}, gated SiLU, "
-            f"recompute={recompute_level.value}",
+            f"recompute={recompute_level.value}, weight-gradient buffers {grad_dtype_name}",
             "tokens": workload.tokens,
             "hidden": hidden,
             "ffn": ffn,
             "experts": workload.experts,
             "experts_per_token": workload.experts_per_token,
+            "grad_dtype": grad_dtype_name,
         },
         "roofline": {
             "bound": "mfma",
             "kernel": "grouped_gemm_mfma_kernel (all grouped-GEMM launches of a step; figures are per launch, averaged over them)",
-            "achieved": gemm_tflops,
-            "peak": PEAK_BF16_TFLOPS,
+            "achieved": timed["gemm_tflops"],
+            "peak": timed["gemm_peak_tflops"],
             "unit": "TFLOP/s",
-            "frac": gemm_tflops / PEAK_BF16_TFLOPS,
+            "frac": timed["gemm_tflops"] / timed["gemm_peak_tflops"],
             "traffic": traffic,
             "traffic_source": traffic_source,
-            "launches_per_step": gemm_launches,
-            "flops_per_launch": gemm_flops / gemm_launches,
-            "ms_per_launch": gemm_ms / gemm_launches,
+            "launches_per_step": timed["gemm_launches"],
+            "flops_per_launch": timed["gemm_flops"] / timed["gemm_launches"],
+            "ms_per_launch": timed["gemm_ms"] / timed["gemm_launches"],
         },
-        "gemm_frac_of_step": gemm_ms / ms_per_step,
-        "kernels": kernels,
+        "gemm_frac_of_step": timed["gemm_ms"] / timed["ms_per_step"],
+        "kernels": timed["kernels"],
     }
+    headline_inputs = timed["inputs"]
+
+    if not args.only:
+        # The same step with the other gradient-buffer layout.
+        other = "same" if args.grad_dtype == "fp32" else "fp32"
+        headline_inputs = None if args.cpu_tokens <= 0 else timed["inputs"].to("cpu")
+        release(timed)
+        other_timed = time_workload(workload, args, args.steps, args.warmup, other, recompute_level, device)
+        release(other_timed)
+        result["other_grad_dtype"] = {
+            "grad_dtype": "f32" if other == "fp32" else dtype_names[workload.dtype],
+            "ms_per_step": round(other_timed["ms_per_step"], 4),
+            "tokens_per_s": round(other_timed["tokens_per_s"], 1),
+            "gemm_tflops": round(other_timed["gemm_tflops"], 1),
+            "gemm_frac": round(other_timed["gemm_tflops"] / other_timed["gemm_peak_tflops"], 4),
+        }
+        # The other configurations: a few steps each, figures per configuration.
+        configs = {workload.name: summary_of(workload, timed)}
+        tiny_inputs = None
+        for name in (HEADLINE,) + OTHER_WORKLOADS:
+            if name == workload.name:
+                continue
+            other_workload = WORKLOADS[name]
+            config_timed = time_workload(other_workload, args, min(args.steps, 10), min(args.warmup, 2), "same",
+                                         recompute_level, device)  # fmt: skip
+            configs[name] = summary_of(other_workload, config_timed)
+            if name == "tiny" and args.cpu_tokens > 0:
+                tiny_inputs = config_timed["inputs"].to("cpu")
+            release(config_timed)
+        result["configs"] = configs
+        if tiny_inputs is not None:
+            result["cpu_baseline_tiny"] = cpu_baseline(WORKLOADS["tiny"], tiny_inputs, WORKLOADS["tiny"].tokens)
     if args.cpu_tokens > 0:
-        result["cpu_baseline"] = cpu_baseline(workload, inputs, min(args.cpu_tokens, workload.tokens))
+        result["cpu_baseline"] = cpu_baseline(workload, headline_inputs, min(args.cpu_tokens, workload.tokens))
     print(json.dumps(result))
 
 

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 7
+#define FM_VERSION 8
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -300,6 +300,21 @@ int fm_output_sparse_matmul_gated_activation_backward(const void *lhs, const voi
                                                       int64_t lhs_stride_inner, int64_t rhs_stride_inner,
                                                       int64_t rhs_stride_col, int activation, int dtype,
                                                       int index_dtype, void *stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Measurement probes (no counterpart in the reference, not on the MoE path): the ceilings the benchmark sets the
+ * kernels' figures against, measured on the device at hand.
+ * --------------------------------------------------------------------------------------------------------- */
+
+/* `workgroups` workgroups of 4 wavefronts each issue `iterations` x 32 back-to-back v_mfma_f32_32x32x16_bf16 from
+ * registers; operands are zeros (random_operands = 0) or normal(0, sigma) values. `sink` receives 256 floats per
+ * workgroup. The work done is fm_probe_mfma_flops(workgroups, iterations). */
+int fm_probe_mfma(void *sink, int64_t workgroups, int64_t iterations, int random_operands, float sigma, void *stream);
+int64_t fm_probe_mfma_flops(int64_t workgroups, int64_t iterations);
+
+/* target[0 .. bytes) = source[0 .. bytes) with 16-byte streaming loads and stores from `workgroups` workgroups of
+ * 256 lanes (grid stride). `bytes` a multiple of 16, both pointers 16-byte aligned. */
+int fm_probe_copy(const void *source, void *target, int64_t bytes, int64_t workgroups, void *stream);
 
 #ifdef __cplusplus
 }

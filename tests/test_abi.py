@@ -20,7 +20,7 @@ def _declared_symbols() -> dict[str, int]:
     """name -> number of parameters, parsed from the header."""
     text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
     symbols = {}
-    for match in re.finditer(r"\b(?:int|size_t|const char \*)\s*(fm_\w+)\s*\(([^)]*)\)\s*;", text):
+    for match in re.finditer(r"\b(?:int|int64_t|size_t|const char \*)\s*(fm_\w+)\s*\(([^)]*)\)\s*;", text):
         params = match.group(2).strip()
         symbols[match.group(1)] = 0 if params in ("", "void") else params.count(",") + 1
     return symbols
