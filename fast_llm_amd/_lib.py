@@ -12,7 +12,7 @@ import torch
 
 LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "csrc" / "libfastmoe_hip.so"
 
-FM_VERSION = 8
+FM_VERSION = 9
 
 _c_i64, _c_int, _c_ptr, _c_size = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
@@ -33,6 +33,11 @@ SIGNATURES: dict[str, tuple] = {
     "fm_topk_routing_backward": (_c_int, [_c_ptr] * 4 + [_c_i64] * 3 + [_c_int, _c_ptr]),
     "fm_router_workspace_size": (_c_size, [_c_i64] * 2),
     "fm_router_forward": (_c_int, [_c_ptr] * 8 + [_c_size] + [_c_i64] * 4 + [_c_int, _c_ptr]),
+    "fm_sparse_map_from_router_workspace_size": (_c_size, [_c_i64] * 2),
+    "fm_sparse_map_from_router": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_size] + [_c_i64] * 5 + [_c_int] + [_c_ptr] * 4 + [_c_size, _c_ptr],
+    ),
     "fm_router_backward": (_c_int, [_c_ptr] * 8 + [ctypes.c_double] * 2 + [_c_i64] * 4 + [_c_int, _c_ptr]),
     "fm_mlp_activation_forward": (_c_int, [_c_ptr] * 2 + [_c_i64] * 2 + [_c_int] * 3 + [_c_ptr, _c_int, _c_ptr]),
     "fm_mlp_activation_backward": (_c_int, [_c_ptr] * 4 + [_c_i64] * 2 + [_c_int] * 3 + [_c_ptr, _c_int, _c_ptr]),

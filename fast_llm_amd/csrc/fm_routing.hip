@@ -7,6 +7,7 @@
 // k rounds of a wave-wide arg-max (ties go to the lower expert index) pick the experts. Latency-bound: the whole
 // input is tokens * experts values.
 #include "fm_common.h"
+#include "fm_router_layout.h"
 
 namespace fm {
 
@@ -108,21 +109,7 @@ __global__ __launch_bounds__(kRoutingThreads) void topk_routing_backward_kernel(
 // A workgroup walks a fixed range of tokens, one wavefront per token, and keeps the per-expert sums of its tokens in
 // registers; the sums of all workgroups are then added in a fixed order by a second kernel, so results do not depend
 // on scheduling.
-struct RouterStats {  // offsets into the statistics array of 2 * experts + 1 floats
-    static __host__ __device__ int probability_sum(int e) { return e; }
-    static __host__ __device__ int count(int experts, int e) { return experts + e; }
-    static __host__ __device__ int z_sum(int experts) { return 2 * experts; }
-    static __host__ __device__ int size(int experts) { return 2 * experts + 1; }
-};
-
 constexpr int kRouterWaves = kRoutingThreads / 64;
-constexpr int kMaxRouterBlocks = 1024;
-constexpr int kRouterTokensPerBlock = 16;
-
-inline int router_blocks(int64_t tokens) {
-    const int64_t blocks = (tokens + kRouterTokensPerBlock - 1) / kRouterTokensPerBlock;
-    return static_cast<int>(blocks < kMaxRouterBlocks ? blocks : kMaxRouterBlocks);
-}
 
 __device__ __forceinline__ float wave_max(float value) {
 #pragma unroll
@@ -168,11 +155,10 @@ __device__ __forceinline__ void load_router_row(const T *logits, const T *noise,
 template <typename T>
 __global__ __launch_bounds__(kRoutingThreads) void router_forward_kernel(
     const T *__restrict__ logits, const T *__restrict__ noise, int64_t *__restrict__ top_experts,
-    float *__restrict__ scores, float *__restrict__ lse, float *__restrict__ partials, int64_t tokens, int experts,
-    int k, int shared) {
+    float *__restrict__ scores, float *__restrict__ lse, float *__restrict__ partials, int64_t tokens,
+    int64_t per_block, int experts, int k, int shared) {
     extern __shared__ float block_sums[];  // [waves][stats]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t per_block = (tokens + gridDim.x - 1) / gridDim.x;
     const int64_t begin = blockIdx.x * per_block, end = min(begin + per_block, tokens);
     const int slots = shared + k;
     float probability_sum[kMaxPerLane], count[kMaxPerLane], z_sum = 0.f;
@@ -426,7 +412,8 @@ extern "C" int fm_router_forward(const void *logits, const void *noise, void *to
         router_forward_kernel<T><<<blocks, kRoutingThreads, sizeof(float) * kRouterWaves * stats, stream>>>(
             static_cast<const T *>(logits), static_cast<const T *>(noise), static_cast<int64_t *>(top_experts),
             static_cast<float *>(scores), static_cast<float *>(lse), static_cast<float *>(workspace), num_tokens,
-            experts, static_cast<int>(experts_per_token), static_cast<int>(shared_experts));
+            router_tokens_per_block(num_tokens), experts, static_cast<int>(experts_per_token),
+            static_cast<int>(shared_experts));
     });
     router_reduce_kernel<<<(stats + kRoutingThreads - 1) / kRoutingThreads, kRoutingThreads, 0, stream>>>(
         static_cast<const float *>(workspace), static_cast<float *>(statistics), blocks, stats);

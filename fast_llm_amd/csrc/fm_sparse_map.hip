@@ -14,6 +14,7 @@
 // Ranks follow the flattened index order, i.e. the order of a stable sort by expert
 // (reference: fast_llm/functional/triton/sparse_copy.py:249-254).
 #include "fm_common.h"
+#include "fm_router_layout.h"
 
 #include <mutex>
 
@@ -60,31 +61,16 @@ __global__ __launch_bounds__(kMapBlock) void sparse_map_histogram_kernel(const i
     for (int e = threadIdx.x; e < num_experts; e += kMapBlock) out[e] = lds_counts[e];
 }
 
-__global__ __launch_bounds__(kMapBlock) void sparse_map_layout_kernel(int32_t *__restrict__ block_counts,
-                                                                      int num_blocks, int num_experts,
-                                                                      int64_t pad_to_multiple, int index_dtype,
-                                                                      void *__restrict__ expert_ends,
-                                                                      void *__restrict__ expert_pad_begins,
-                                                                      int32_t *__restrict__ expert_begins) {
+// Second half of the layout kernels: thread e holds count[e]; writes expert_ends, expert_pad_begins and the first row
+// of every expert (inclusive scan of the padded counts over experts: wavefront scan, then the wavefront totals).
+__device__ __forceinline__ void write_expert_layout(int64_t count, int num_experts, int64_t pad_to_multiple,
+                                                    int index_dtype, void *__restrict__ expert_ends,
+                                                    void *__restrict__ expert_pad_begins,
+                                                    int32_t *__restrict__ expert_begins) {
     __shared__ int64_t lds_wave_totals[kMapWaves];
     const int e = threadIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-
-    // Exclusive prefix over workgroups of this expert's counts, in place.
-    int64_t count = 0;
-    if (e < num_experts) {
-        int32_t running = 0;
-        for (int b = 0; b < num_blocks; ++b) {
-            int32_t *slot = block_counts + static_cast<int64_t>(b) * num_experts + e;
-            const int32_t here = *slot;
-            *slot = running;
-            running += here;
-        }
-        count = running;
-    }
     const int64_t padded = (count + pad_to_multiple - 1) / pad_to_multiple * pad_to_multiple;
-
-    // Inclusive scan of `padded` over experts: wavefront scan, then the wavefront totals.
     int64_t inclusive = padded;
 #pragma unroll
     for (int offset = 1; offset < 64; offset <<= 1) {
@@ -105,45 +91,106 @@ __global__ __launch_bounds__(kMapBlock) void sparse_map_layout_kernel(int32_t *_
     }
 }
 
+__global__ __launch_bounds__(kMapBlock) void sparse_map_layout_kernel(int32_t *__restrict__ block_counts,
+                                                                      int num_blocks, int num_experts,
+                                                                      int64_t pad_to_multiple, int index_dtype,
+                                                                      void *__restrict__ expert_ends,
+                                                                      void *__restrict__ expert_pad_begins,
+                                                                      int32_t *__restrict__ expert_begins) {
+    const int e = threadIdx.x;
+    // Exclusive prefix over workgroups of this expert's counts, in place.
+    int64_t count = 0;
+    if (e < num_experts) {
+        int32_t running = 0;
+        for (int b = 0; b < num_blocks; ++b) {
+            int32_t *slot = block_counts + static_cast<int64_t>(b) * num_experts + e;
+            const int32_t here = *slot;
+            *slot = running;
+            running += here;
+        }
+        count = running;
+    }
+    write_expert_layout(count, num_experts, pad_to_multiple, index_dtype, expert_ends, expert_pad_begins, expert_begins);
+}
+
+// The same from what the router's forward kernel left in its workspace: per workgroup of that kernel (a fixed range
+// of `tokens_per_block` tokens) and routed expert, the number of tokens of the range that selected the expert, as a
+// float (exact: at most 2^24). Shared experts follow the routed ones and are selected by every token.
+__global__ __launch_bounds__(kMapBlock) void sparse_map_layout_from_router_kernel(
+    const float *__restrict__ router_partials, int router_stats, int num_blocks, int64_t num_tokens,
+    int64_t tokens_per_block, int routed_experts, int num_experts, int64_t pad_to_multiple, int index_dtype,
+    void *__restrict__ expert_ends, void *__restrict__ expert_pad_begins, int32_t *__restrict__ block_prefix,
+    int32_t *__restrict__ expert_begins) {
+    const int e = threadIdx.x;
+    int64_t count = 0;
+    if (e < num_experts) {
+        int32_t running = 0;
+        for (int b = 0; b < num_blocks; ++b) {
+            int32_t here;
+            if (e < routed_experts) {
+                here = static_cast<int32_t>(router_partials[static_cast<int64_t>(b) * router_stats + routed_experts + e]);
+            } else {
+                const int64_t begin = b * tokens_per_block;
+                here = static_cast<int32_t>(max(int64_t(0), min(begin + tokens_per_block, num_tokens) - begin));
+            }
+            block_prefix[static_cast<int64_t>(b) * num_experts + e] = running;
+            running += here;
+        }
+        count = running;
+    }
+    write_expert_layout(count, num_experts, pad_to_multiple, index_dtype, expert_ends, expert_pad_begins, expert_begins);
+}
+
+// Workgroup b ranks the entries [b * entries_per_block, (b + 1) * entries_per_block) of the flattened `top_experts`,
+// 1024 at a time, given the number of earlier entries per expert (`block_prefix[b]`).
 __global__ __launch_bounds__(kMapBlock) void sparse_map_rows_kernel(const int64_t *__restrict__ top_experts,
-                                                                    int64_t num_entries, int num_experts,
+                                                                    int64_t num_entries, int64_t entries_per_block,
+                                                                    int num_experts,
                                                                     const int32_t *__restrict__ block_prefix,
                                                                     const int32_t *__restrict__ expert_begins,
                                                                     int index_dtype, void *__restrict__ sparse_rows) {
-    extern __shared__ int32_t lds_wave_counts[];  // [kMapWaves][num_experts]
-    for (int i = threadIdx.x; i < kMapWaves * num_experts; i += kMapBlock) lds_wave_counts[i] = 0;
-    __syncthreads();
-
-    const int64_t entry = static_cast<int64_t>(blockIdx.x) * kMapBlock + threadIdx.x;
-    int64_t expert64 = entry < num_entries ? top_experts[entry] : -1;
-    const bool valid = expert64 >= 0 && expert64 < num_experts;
-    const int expert = valid ? static_cast<int>(expert64) : 0;
-    const uint64_t same = match_expert(expert, valid, log2_ceil(num_experts));
+    extern __shared__ int32_t lds_map[];  // [kMapWaves][num_experts] counts per wavefront, then [num_experts] running
+    int32_t *lds_wave_counts = lds_map;
+    int32_t *lds_running = lds_map + kMapWaves * num_experts;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int rank_in_wave = __popcll(same & ((1ull << lane) - 1));
-    if (valid && rank_in_wave == 0) lds_wave_counts[wave * num_experts + expert] = __popcll(same);
-    __syncthreads();
+    const int num_bits = log2_ceil(num_experts);
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * entries_per_block;
+    const int64_t last = min(first + entries_per_block, num_entries);
+    for (int e = threadIdx.x; e < num_experts; e += kMapBlock)
+        lds_running[e] = expert_begins[e] + block_prefix[static_cast<int64_t>(blockIdx.x) * num_experts + e];
 
-    // Exclusive prefix over the wavefronts of the workgroup, per expert, in place.
-    for (int e = threadIdx.x; e < num_experts; e += kMapBlock) {
-        int32_t running = 0;
+    for (int64_t chunk = first; chunk < last; chunk += kMapBlock) {
+        for (int i = threadIdx.x; i < kMapWaves * num_experts; i += kMapBlock) lds_wave_counts[i] = 0;
+        __syncthreads();
+
+        const int64_t entry = chunk + threadIdx.x;
+        int64_t expert64 = entry < last ? top_experts[entry] : -1;
+        const bool valid = expert64 >= 0 && expert64 < num_experts;
+        const int expert = valid ? static_cast<int>(expert64) : 0;
+        const uint64_t same = match_expert(expert, valid, num_bits);
+        const int rank_in_wave = __popcll(same & ((1ull << lane) - 1));
+        if (valid && rank_in_wave == 0) lds_wave_counts[wave * num_experts + expert] = __popcll(same);
+        __syncthreads();
+
+        // Exclusive prefix over the wavefronts of the workgroup, per expert, in place, on top of the running count.
+        for (int e = threadIdx.x; e < num_experts; e += kMapBlock) {
+            int32_t running = lds_running[e];
 #pragma unroll
-        for (int w = 0; w < kMapWaves; ++w) {
-            const int32_t here = lds_wave_counts[w * num_experts + e];
-            lds_wave_counts[w * num_experts + e] = running;
-            running += here;
+            for (int w = 0; w < kMapWaves; ++w) {
+                const int32_t here = lds_wave_counts[w * num_experts + e];
+                lds_wave_counts[w * num_experts + e] = running;
+                running += here;
+            }
+            lds_running[e] = running;
         }
-    }
-    __syncthreads();
+        __syncthreads();
 
-    if (entry < num_entries) {
-        int64_t row = -1;
-        if (valid) {
-            row = static_cast<int64_t>(expert_begins[expert]) +
-                  block_prefix[static_cast<int64_t>(blockIdx.x) * num_experts + expert] +
-                  lds_wave_counts[wave * num_experts + expert] + rank_in_wave;
+        if (entry < last) {
+            int64_t row = -1;
+            if (valid) row = static_cast<int64_t>(lds_wave_counts[wave * num_experts + expert]) + rank_in_wave;
+            store_index(sparse_rows, index_dtype, entry, row);
         }
-        store_index(sparse_rows, index_dtype, entry, row);
+        __syncthreads();
     }
 }
 
@@ -179,8 +226,8 @@ static int run_sparse_map(const char *name, const int64_t *top_experts, int64_t 
     sparse_map_layout_kernel<<<1, kMapBlock, 0, stream>>>(block_counts, blocks, experts, pad_to_multiple, index_dtype,
                                                           expert_ends, expert_pad_begins, expert_begins);
     if (blocks > 0) {
-        sparse_map_rows_kernel<<<blocks, kMapBlock, kMapWaves * experts * sizeof(int32_t), stream>>>(
-            top_experts, num_entries, experts, block_counts, expert_begins, index_dtype, sparse_rows);
+        sparse_map_rows_kernel<<<blocks, kMapBlock, (kMapWaves + 1) * experts * sizeof(int32_t), stream>>>(
+            top_experts, num_entries, kMapBlock, experts, block_counts, expert_begins, index_dtype, sparse_rows);
     }
     return check_launch(name);
 }
@@ -221,6 +268,52 @@ extern "C" int fm_sparse_map(const int64_t *top_experts, int64_t num_rows_dense,
     return run_sparse_map("fm_sparse_map", top_experts, num_rows_dense, num_experts_per_token, num_experts,
                           pad_to_multiple, index_dtype, sparse_rows, expert_ends, expert_pad_begins, workspace,
                           static_cast<hipStream_t>(stream));
+}
+
+// ---- the map from the router's own counts ------------------------------------------------------------------
+extern "C" size_t fm_sparse_map_from_router_workspace_size(int64_t num_tokens, int64_t num_experts) {
+    if (num_tokens < 0 || num_experts < 0) return 0;
+    const size_t bytes = static_cast<size_t>(fm::router_blocks(num_tokens) + 1) * num_experts * sizeof(int32_t);
+    return (bytes + 255) / 256 * 256 + 256;
+}
+
+extern "C" int fm_sparse_map_from_router(const int64_t *top_experts, const void *router_workspace,
+                                         size_t router_workspace_size, int64_t num_tokens, int64_t num_experts,
+                                         int64_t experts_per_token, int64_t shared_experts, int64_t pad_to_multiple,
+                                         int index_dtype, void *sparse_rows, void *expert_ends,
+                                         void *expert_pad_begins, void *workspace, size_t workspace_size,
+                                         void *stream_) {
+    using namespace fm;
+    const char *name = "fm_sparse_map_from_router";
+    FM_REQUIRE(shared_experts >= 0 && experts_per_token > 0 && num_experts > shared_experts,
+               "%s: %lld experts of which %lld shared, %lld per token", name, (long long)num_experts,
+               (long long)shared_experts, (long long)experts_per_token);
+    const int64_t slots = shared_experts + experts_per_token, routed = num_experts - shared_experts;
+    if (int status = check_sparse_map_arguments(name, top_experts, num_tokens, slots, num_experts, pad_to_multiple,
+                                                index_dtype, sparse_rows, expert_ends, expert_pad_begins))
+        return status;
+    FM_REQUIRE(num_tokens > 0, "%s: no tokens (the router does not run on none either)", name);
+    const int blocks = router_blocks(num_tokens);
+    const int stats = RouterStats::size(static_cast<int>(routed));
+    FM_REQUIRE(router_workspace && router_workspace_size >= sizeof(float) * blocks * stats,
+               "%s: the router workspace must be the %zu bytes fm_router_forward filled, got %zu", name,
+               sizeof(float) * blocks * stats, router_workspace_size);
+    FM_REQUIRE(workspace && aligned16(workspace) &&
+                   workspace_size >= fm_sparse_map_from_router_workspace_size(num_tokens, num_experts),
+               "%s: workspace of %zu bytes is null, misaligned or too small", name, workspace_size);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int experts = static_cast<int>(num_experts);
+    const int64_t tokens_per_block = router_tokens_per_block(num_tokens);
+    int32_t *block_prefix = static_cast<int32_t *>(workspace);
+    int32_t *expert_begins = block_prefix + static_cast<int64_t>(blocks) * experts;
+    sparse_map_layout_from_router_kernel<<<1, kMapBlock, 0, stream>>>(
+        static_cast<const float *>(router_workspace), stats, blocks, num_tokens, tokens_per_block,
+        static_cast<int>(routed), experts, pad_to_multiple, index_dtype, expert_ends, expert_pad_begins, block_prefix,
+        expert_begins);
+    sparse_map_rows_kernel<<<blocks, kMapBlock, (kMapWaves + 1) * experts * sizeof(int32_t), stream>>>(
+        top_experts, num_tokens * slots, tokens_per_block * slots, experts, block_prefix, expert_begins, index_dtype,
+        sparse_rows);
+    return check_launch(name);
 }
 
 // ---- the same map without any allocation ----------------------------------------------------------------

@@ -42,11 +42,15 @@ def get_sparse_map(
     pad_to_multiple: int = MAX_DROPLESS_BLOCK_SIZE_ROW,
     block_size=KernelConfig.POINTWISE_BLOCK_SIZE,
     use_triton: bool | None = None,
+    router_counts=None,
 ) -> SparseMap:
     """
     Expert histogram, padded expert offsets and the stable sparse row of every (token, slot).
     Reference: fast_llm/functional/triton/sparse_copy.py:258-301 (`block_size` is a Triton launch parameter there and
     has no effect here; `use_triton=False` selects the reference's torch path, which this package does not have).
+    `router_counts` (not in the reference's signature): the `RouterCounts` that `functional.routing.router` returned
+    together with these very `top_experts`; the map is then built from the router's counts, without the pass that
+    counts `top_experts`. Same result.
     """
     KernelConfig.enabled(top_experts.device, use_triton)
     Assert.eq(top_experts.dim(), 2)
@@ -61,6 +65,35 @@ def get_sparse_map(
     expert_ends = torch.empty(num_experts, dtype=dtype, device=device)
     expert_pad_begins = torch.empty(num_experts, dtype=dtype, device=device)
     library = _lib.lib()
+    if router_counts is not None:
+        Assert.eq(router_counts.tokens, num_rows_dense)
+        Assert.eq(router_counts.shared_experts + router_counts.experts_per_token, num_experts_per_token)
+        Assert.eq(router_counts.shared_experts + router_counts.routed_experts, num_experts)
+        _lib.require_device(top_experts, router_counts.workspace)
+        workspace_size = library.fm_sparse_map_from_router_workspace_size(num_rows_dense, num_experts)
+        workspace = torch.empty(workspace_size, dtype=torch.uint8, device=device)
+        _lib.call(
+            "fm_sparse_map_from_router",
+            device,
+            _lib.ptr(top_experts),
+            _lib.ptr(router_counts.workspace),
+            router_counts.workspace.numel() * router_counts.workspace.element_size(),
+            num_rows_dense,
+            num_experts,
+            router_counts.experts_per_token,
+            router_counts.shared_experts,
+            pad_to_multiple,
+            _lib.index_tag(dtype),
+            _lib.ptr(sparse_rows),
+            _lib.ptr(expert_ends),
+            _lib.ptr(expert_pad_begins),
+            _lib.ptr(workspace),
+            workspace_size,
+            label="fm_sparse_map",
+        )
+        return _finish_sparse_map(
+            sparse_rows, expert_ends, expert_pad_begins, num_experts, dynamic_shape, max_rows
+        )
     workspace_size = library.fm_sparse_map_workspace_size(num_rows_dense, num_experts_per_token, num_experts)
     workspace = torch.empty(workspace_size, dtype=torch.uint8, device=device)
     _lib.call(
@@ -78,13 +111,25 @@ def get_sparse_map(
         _lib.ptr(workspace),
         workspace_size,
     )
+    return _finish_sparse_map(sparse_rows, expert_ends, expert_pad_begins, num_experts, dynamic_shape, max_rows)
+
+
+def _finish_sparse_map(
+    sparse_rows: torch.Tensor,
+    expert_ends: torch.Tensor,
+    expert_pad_begins: torch.Tensor,
+    num_experts: int,
+    dynamic_shape: bool,
+    max_rows: int,
+) -> SparseMap:
+    num_rows_dense, num_experts_per_token = sparse_rows.shape
     return SparseMap(
         sparse_rows=sparse_rows,
         expert_ends=expert_ends,
         expert_pad_begins=expert_pad_begins,
         num_rows_dense=num_rows_dense,
         num_rows=expert_ends[-1].item() if dynamic_shape else max_rows,
-        num_rows_unpadded=num_rows_unpadded,
+        num_rows_unpadded=num_rows_dense * num_experts_per_token,
         num_experts=num_experts,
         num_experts_per_token=num_experts_per_token,
     )

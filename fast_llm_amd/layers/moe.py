@@ -60,6 +60,7 @@ class DroplessMoEMLP(torch.nn.Module):
         self.jitter_eps = jitter_eps
         self.gated, self.activation = gated, activation
         self.recompute_level, self.dropless_dynamic_shape = recompute_level, dropless_dynamic_shape
+        self._router_counts = None
         layer_1_rows = experts * intermediate_size * (2 if gated else 1)
         self.router = torch.nn.Parameter(torch.empty(self.unshared_experts, hidden_size, dtype=dtype, device=device))
         self.layer_1 = torch.nn.Parameter(torch.empty(layer_1_rows, hidden_size, dtype=dtype, device=device))
@@ -84,13 +85,14 @@ class DroplessMoEMLP(torch.nn.Module):
         if self.training and self.jitter_eps > 0.0:
             noise = torch.empty_like(logits).uniform_(1.0 - self.jitter_eps, 1.0 + self.jitter_eps)
         trained = self.training and grad_scale is not None
-        scores, top_experts, load_balancing_loss, z_loss = router(
+        scores, top_experts, load_balancing_loss, z_loss, self._router_counts = router(
             logits,
             self.experts_per_token,
             shared_experts=self.shared_experts,
             noise=noise,
             auxiliary_loss_grad=self.unshared_experts * self.auxiliary_loss_coefficient * grad_scale if trained else None,
             z_loss_grad=self.z_loss_coefficient * grad_scale if trained else None,
+            return_counts=True,
         )
         if losses is not None:
             losses.setdefault(LOAD_BALANCING_LOSS, []).append(load_balancing_loss)
@@ -109,9 +111,14 @@ class DroplessMoEMLP(torch.nn.Module):
     ) -> torch.Tensor:
         """`scores`/`top_experts` may be passed to bypass the router (tests pin the routing that way)."""
         hidden_states = input_.flatten(0, -2)
+        router_counts = None
         if top_experts is None:
             scores, top_experts = self.route(hidden_states, grad_scale, losses)
-        sparse_map = get_sparse_map(top_experts, self.experts, dynamic_shape=self.dropless_dynamic_shape)
+            # The router has counted the tokens of every expert on its way: the map need not count them again.
+            router_counts, self._router_counts = self._router_counts, None
+        sparse_map = get_sparse_map(
+            top_experts, self.experts, dynamic_shape=self.dropless_dynamic_shape, router_counts=router_counts
+        )
         output = mlp_autograd(
             hidden_states,
             scores,

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 8
+#define FM_VERSION 9
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -190,6 +190,21 @@ int fm_router_backward(const void *grad_scores, const void *scores, const void *
                        const void *noise, const void *lse, const void *statistics, void *grad_logits,
                        double auxiliary_loss_grad, double z_loss_grad, int64_t num_tokens, int64_t num_experts,
                        int64_t experts_per_token, int64_t shared_experts, int dtype, void *stream);
+
+/* The sparse map from the router's own counts: `fm_router_forward` has already counted, per workgroup of its kernel,
+ * how many tokens selected each routed expert, and left the counts in its workspace. Given that workspace unmodified
+ * (same num_tokens; num_experts here counts routed + shared experts), this builds the map of `top_experts`
+ * [num_tokens, shared_experts + experts_per_token] without the counting pass over `top_experts`. Same results as
+ * `fm_sparse_map(top_experts, num_tokens, shared_experts + experts_per_token, num_experts, ...)`, bit for bit.
+ * Replaces the same reference lines as `fm_sparse_map`, for the caller
+ * fast_llm/layers/decoder/mlp/mixture_of_experts.py:163-171, 193-196 (routing followed by `get_sparse_map`).
+ * `workspace`: fm_sparse_map_from_router_workspace_size(num_tokens, num_experts) bytes, 16-byte aligned. */
+size_t fm_sparse_map_from_router_workspace_size(int64_t num_tokens, int64_t num_experts);
+int fm_sparse_map_from_router(const int64_t *top_experts, const void *router_workspace, size_t router_workspace_size,
+                              int64_t num_tokens, int64_t num_experts, int64_t experts_per_token,
+                              int64_t shared_experts, int64_t pad_to_multiple, int index_dtype, void *sparse_rows,
+                              void *expert_ends, void *expert_pad_begins, void *workspace, size_t workspace_size,
+                              void *stream);
 
 /* ---------------------------------------------------------------------------------------------------------
  * MLP activation. `input` is [num_rows, num_columns * (gated ? 2 : 1)], `output`/`grad_output` are

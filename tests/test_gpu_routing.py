@@ -236,3 +236,40 @@ def test_router_with_masked_experts_and_full_selection(device):
     assert torch.equal(top_experts.cpu().sort(dim=-1).values, torch.arange(6).expand(64, 6))
     full = torch.softmax(logits, dim=-1)
     assert torch.allclose(scores.cpu(), full.gather(1, top_experts.cpu()), rtol=2e-6, atol=1e-7)
+
+
+# (tokens, routed experts, k, shared): the five benchmark configurations' routers, shared experts, token counts that
+# leave the router's last workgroups short or empty, more than 1024 x 16 tokens (several map chunks per workgroup),
+# and slot counts that do not divide the map kernel's chunk of 1024 entries.
+_HANDOFF_CASES = [
+    (512, 8, 2, 0), (8192, 8, 2, 0), (16384, 64, 6, 0), (16384, 128, 8, 0), (8192, 8, 2, 2), (100, 6, 3, 1),
+    (1, 4, 2, 0), (17, 5, 5, 3), (40000, 16, 7, 1), (70001, 1000, 3, 0), (5627, 60, 56, 8),
+]  # fmt: skip
+
+
+@pytest.mark.parametrize(("tokens", "experts", "k", "shared"), _HANDOFF_CASES)
+@pytest.mark.parametrize("zipf", [False, True])
+def test_sparse_map_from_the_routers_counts(tokens, experts, k, shared, zipf, device):
+    """The router already counts the tokens of every expert; the map built from those counts (no counting pass over
+    `top_experts`) equals the map built from `top_experts` alone and the oracle's map, bit for bit."""
+    from fast_llm_amd.functional.sparse_copy import get_sparse_map
+
+    generator = torch.Generator().manual_seed(tokens + 31 * experts + shared)
+    logits = torch.randn(tokens, experts, generator=generator)
+    if zipf:  # load imbalance, near-empty experts
+        logits += 3 * torch.log(torch.arange(1, experts + 1, dtype=torch.float32) ** -1.2)
+    scores, top_experts, _, _, counts = router(logits.to(device), k, shared_experts=shared, return_counts=True)
+    total = experts + shared
+    handed = get_sparse_map(top_experts, total, router_counts=counts)
+    counted = get_sparse_map(top_experts, total)
+    expected = moe_oracle.sparse_map(top_experts.cpu(), total)
+    for name in ("sparse_rows", "expert_ends", "expert_pad_begins"):
+        ours = getattr(handed, name)
+        assert ours.dtype == getattr(counted, name).dtype
+        assert torch.equal(ours, getattr(counted, name)), name
+        assert torch.equal(ours.cpu().long(), getattr(expected, name)), name
+    assert handed.num_rows == counted.num_rows == expected.num_rows
+    with pytest.raises(AssertionError):  # counts of another routing
+        get_sparse_map(top_experts[: tokens // 2 + 1], total, router_counts=counts) if tokens > 1 else get_sparse_map(
+            top_experts, total + 1, router_counts=counts
+        )
