@@ -208,3 +208,41 @@ def router(
     if return_counts:
         result += (RouterCounts(workspace, flat.size(0), flat.size(1), experts_per_token, shared_experts),)
     return result
+
+
+def sinkhorn(cost: torch.Tensor, tolerance: float = 1e-5, eps: float = 1e-9) -> torch.Tensor:
+    """Sinkhorn normalisation of exp(cost): alternately rescales rows and columns until the column scales move by less
+    than `tolerance` on average; rows of the result sum to 1 / tokens, columns to about 1 / experts. No gradient.
+    Reference: fast_llm/layers/decoder/mlp/mixture_of_experts.py:389-403 (a data-dependent number of small torch
+    reductions over [tokens, experts]; it is upstream of the dropless path and stays in torch)."""
+    with torch.no_grad():
+        cost = torch.exp(cost.to(torch.float32))
+        d0 = torch.ones(cost.shape[:-1], device=cost.device, dtype=cost.dtype)
+        d1 = torch.ones(cost.shape[-1:], device=cost.device, dtype=cost.dtype)
+        error = eps**-1
+        d1_old = d1
+        while error > tolerance:
+            d0 = d0.numel() ** -1 / (torch.sum(d1 * cost, -1) + eps)
+            d1 = d1.numel() ** -1 / (torch.sum((d0.unsqueeze(-1) * cost).flatten(0, -2), 0) + eps)
+            error = torch.mean(torch.abs(d1_old - d1))
+            d1_old = d1
+        return d1 * cost * d0.unsqueeze(-1)
+
+
+def sinkhorn_routing(logits: torch.Tensor, experts_per_token: int, training: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    """(scores, top_experts) of the reference's sinkhorn routing (mixture_of_experts.py:280-296): when training, the
+    experts are the top-k of the sinkhorn-balanced logits and the scores are the activated logits gathered there;
+    otherwise top-k of the activated logits. The activation is a sigmoid for one expert per token, else an fp32
+    softmax cast back to the logits' dtype."""
+
+    def activation(x: torch.Tensor) -> torch.Tensor:
+        if experts_per_token == 1:
+            return torch.sigmoid(x)
+        return torch.softmax(x, dim=-1, dtype=torch.float32).type_as(x)
+
+    if training:
+        _, top_experts = torch.topk(sinkhorn(logits), k=experts_per_token, dim=-1)
+        scores = torch.gather(activation(logits), -1, top_experts)
+    else:
+        scores, top_experts = torch.topk(activation(logits), k=experts_per_token, dim=-1)
+    return scores, top_experts

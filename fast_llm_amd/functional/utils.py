@@ -63,3 +63,17 @@ def wrap_forward_backward(
         return Function.apply(*args, *kwargs.values(), in_)
 
     return call
+
+
+class AuxiliaryLoss(torch.autograd.Function):
+    """Identity on `input_` whose backward also hands the constant `grad` to `aux_loss`: attaches an auxiliary loss
+    to the graph at the tensor it regularises. Reference: fast_llm/functional/utils.py:63-71."""
+
+    @staticmethod
+    def forward(ctx, input_: torch.Tensor, aux_loss: torch.Tensor, grad: float | None) -> torch.Tensor:  # noqa
+        ctx.grad = None if grad is None else torch.full_like(aux_loss, grad)
+        return input_
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor) -> tuple[torch.Tensor | None, ...]:  # noqa
+        return grad_output, ctx.grad, None

@@ -23,9 +23,11 @@ def attach_grad_buffer(weight: torch.Tensor, dtype: torch.dtype | None = None) -
     return weight
 
 
-from fast_llm_amd.functional.routing import router, topk_routing  # noqa: E402, F401  (re-exported)
+from fast_llm_amd.functional.routing import router, sinkhorn_routing, topk_routing  # noqa: E402, F401  (re-exported)
+from fast_llm_amd.functional.utils import AuxiliaryLoss  # noqa: E402
 
 LOAD_BALANCING_LOSS, ROUTER_Z_LOSS = "load_balancing_loss", "router_z_loss"  # layers/decoder/mlp/config.py:24-26
+ROUTING_TOPK, ROUTING_SINKHORN = "aux_loss", "sinkhorn"  # `RoutingType`, layers/decoder/mlp/config.py:29-31
 
 
 class DroplessMoEMLP(torch.nn.Module):
@@ -44,6 +46,11 @@ class DroplessMoEMLP(torch.nn.Module):
         auxiliary_loss_coefficient: float = 0.01,
         z_loss_coefficient: float = 0.0,
         jitter_eps: float = 0.0,
+        routing: str = ROUTING_TOPK,
+        router_normalization: torch.nn.Module | None = None,
+        router_scale: bool = False,
+        router_input_scale: float = 1.0,
+        router_per_expert_scale: bool = False,
         full_precision_gradients: bool = False,
         init_std: float = 0.02,
         dtype: torch.dtype = torch.bfloat16,
@@ -58,6 +65,23 @@ class DroplessMoEMLP(torch.nn.Module):
         self.unshared_experts = experts - shared_experts
         self.auxiliary_loss_coefficient, self.z_loss_coefficient = auxiliary_loss_coefficient, z_loss_coefficient
         self.jitter_eps = jitter_eps
+        if routing not in (ROUTING_TOPK, ROUTING_SINKHORN):
+            raise NotImplementedError(routing)
+        if routing == ROUTING_SINKHORN and shared_experts:
+            # The reference appends the shared experts on the top-k branch only (mixture_of_experts.py:163-168).
+            raise ValueError("sinkhorn routing has no shared experts")
+        self.routing = routing
+        # The router's own view of the input (layers/decoder/mlp/config.py:101-122; mixture_of_experts.py:83-105,
+        # 130-145): an optional normalisation layer, a learnable per-feature scale, a constant, and after the
+        # routing a learnable per-expert scale on the scores. All upstream of the kernels: plain torch modules.
+        self.router_normalization = router_normalization
+        self.router_input_scale = router_input_scale
+        self.router_scale = (
+            torch.nn.Parameter(torch.ones(hidden_size, dtype=dtype, device=device)) if router_scale else None
+        )
+        self.router_per_expert_scale = (
+            torch.nn.Parameter(torch.ones(experts, dtype=dtype, device=device)) if router_per_expert_scale else None
+        )
         self.gated, self.activation = gated, activation
         self.recompute_level, self.dropless_dynamic_shape = recompute_level, dropless_dynamic_shape
         self._router_counts = None
@@ -80,11 +104,18 @@ class DroplessMoEMLP(torch.nn.Module):
         """Router logits to (scores, top_experts), shared experts included. `grad_scale` (the reference's
         `kwargs["grad_output"]`) makes the two auxiliary losses train the router; `losses` collects their values
         (mixture_of_experts.py:146-171, 237-262)."""
-        logits = torch.nn.functional.linear(hidden_states, self.router)
+        router_input = hidden_states if self.router_normalization is None else self.router_normalization(hidden_states)
+        if self.router_scale is not None:
+            router_input = router_input * self.router_scale
+        if self.router_input_scale != 1.0:
+            router_input = router_input * self.router_input_scale
+        logits = torch.nn.functional.linear(router_input, self.router)
         noise = None
         if self.training and self.jitter_eps > 0.0:
             noise = torch.empty_like(logits).uniform_(1.0 - self.jitter_eps, 1.0 + self.jitter_eps)
         trained = self.training and grad_scale is not None
+        if self.routing == ROUTING_SINKHORN:
+            return self._scale_per_expert(*self._route_sinkhorn(logits, noise, grad_scale if trained else None, losses))
         scores, top_experts, load_balancing_loss, z_loss, self._router_counts = router(
             logits,
             self.experts_per_token,
@@ -98,7 +129,27 @@ class DroplessMoEMLP(torch.nn.Module):
             losses.setdefault(LOAD_BALANCING_LOSS, []).append(load_balancing_loss)
             if self.z_loss_coefficient > 0.0:
                 losses.setdefault(ROUTER_Z_LOSS, []).append(z_loss)
+        return self._scale_per_expert(scores, top_experts)
+
+    def _scale_per_expert(self, scores: torch.Tensor, top_experts: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        if self.router_per_expert_scale is not None:  # mixture_of_experts.py:174-175
+            scores = scores * self.router_per_expert_scale[top_experts]
         return scores, top_experts
+
+    def _route_sinkhorn(
+        self, logits: torch.Tensor, noise: torch.Tensor | None, grad_scale: float | None, losses: dict | None
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """z-loss, jitter and sinkhorn routing as the reference orders them (mixture_of_experts.py:146-171)."""
+        self._router_counts = None
+        if self.z_loss_coefficient > 0.0 and (grad_scale is not None or losses is not None):
+            loss = torch.mean(torch.logsumexp(logits.float(), dim=-1) ** 2)
+            if losses is not None:
+                losses.setdefault(ROUTER_Z_LOSS, []).append(loss.detach())
+            if grad_scale is not None:
+                logits = AuxiliaryLoss.apply(logits, loss, self.z_loss_coefficient * grad_scale)
+        if noise is not None:
+            logits = logits * noise
+        return sinkhorn_routing(logits, self.experts_per_token, self.training)
 
     def forward(
         self,

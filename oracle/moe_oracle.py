@@ -503,3 +503,54 @@ def router_backward(
     )
     (grad_logits,) = torch.autograd.grad(total, logits)
     return grad_logits
+
+
+def router_input(
+    hidden_states: torch.Tensor,
+    normalization: typing.Callable[[torch.Tensor], torch.Tensor] | None = None,
+    scale: torch.Tensor | None = None,
+    input_scale: float = 1.0,
+) -> torch.Tensor:
+    """What the router's linear layer sees (fast_llm/layers/decoder/mlp/mixture_of_experts.py:123-145): the hidden
+    states through the optional router normalisation, times the optional per-feature scale, times the constant."""
+    x = hidden_states if normalization is None else normalization(hidden_states)
+    if scale is not None:
+        x = x * scale
+    if input_scale != 1.0:
+        x = x * input_scale
+    return x
+
+
+def per_expert_scale(scores: torch.Tensor, top_experts: torch.Tensor, scale: torch.Tensor | None) -> torch.Tensor:
+    """scores * scale[top_experts] (mixture_of_experts.py:174-175)."""
+    return scores if scale is None else scores * scale[top_experts]
+
+
+def sinkhorn(cost: torch.Tensor, tolerance: float = 1e-5, eps: float = 1e-9) -> torch.Tensor:
+    """The reference's sinkhorn iteration (mixture_of_experts.py:389-403) with explicit sums: row scales
+    d0[t] = (1 / T) / (sum_e d1[e] c[t, e] + eps), column scales d1[e] = (1 / E) / (sum_t d0[t] c[t, e] + eps),
+    c = exp(cost), repeated until mean |d1 - d1_previous| <= tolerance; returns d0[t] c[t, e] d1[e]."""
+    c = torch.exp(cost.to(torch.float32))
+    tokens, experts = c.shape
+    d0, d1 = torch.ones(tokens), torch.ones(experts)
+    while True:
+        d0 = (1.0 / tokens) / ((c * d1[None, :]).sum(dim=1) + eps)
+        new_d1 = (1.0 / experts) / ((c * d0[:, None]).sum(dim=0) + eps)
+        error = (new_d1 - d1).abs().mean().item()
+        d1 = new_d1
+        if not error > tolerance:
+            break
+    return d0[:, None] * c * d1[None, :]
+
+
+def sinkhorn_routing(logits: torch.Tensor, experts_per_token: int, training: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    """(scores, top_experts) of `_sinkhorn_routing` (mixture_of_experts.py:280-296)."""
+    if experts_per_token == 1:
+        activated = torch.sigmoid(logits)
+    else:
+        activated = torch.softmax(logits, dim=-1, dtype=torch.float32).type_as(logits)
+    if training:
+        top_experts = torch.topk(sinkhorn(logits.detach()), k=experts_per_token, dim=-1).indices
+        return torch.gather(activated, -1, top_experts), top_experts
+    scores, top_experts = torch.topk(activated, k=experts_per_token, dim=-1)
+    return scores, top_experts

@@ -273,3 +273,93 @@ def test_sparse_map_from_the_routers_counts(tokens, experts, k, shared, zipf, de
         get_sparse_map(top_experts[: tokens // 2 + 1], total, router_counts=counts) if tokens > 1 else get_sparse_map(
             top_experts, total + 1, router_counts=counts
         )
+
+
+def _rms_norm(hidden: int, device) -> torch.nn.Module:
+    class RMSNorm(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.rand(hidden, device=device) + 0.5)
+
+        def forward(self, x):
+            return x * torch.rsqrt((x.float() ** 2).mean(-1, keepdim=True) + 1e-5).to(x.dtype) * self.weight
+
+    return RMSNorm()
+
+
+@pytest.mark.parametrize("routing", ["aux_loss", "sinkhorn"])
+@pytest.mark.parametrize("training", [True, False])
+def test_layer_with_router_input_options(routing, training, device):
+    """The router's own view of the input (normalisation layer, per-feature scale, constant), the per-expert scale on
+    the scores and sinkhorn routing (fast_llm/layers/decoder/mlp/config.py:101-122, 147-151;
+    mixture_of_experts.py:130-175, 280-296): the whole block against the oracle's restatement of those steps followed by
+    its per-expert loop, gradients down to every router-side parameter by torch autograd of the restatement."""
+    from fast_llm_amd.layers.moe import DroplessMoEMLP
+
+    torch.manual_seed(7)
+    tokens, hidden, ffn, experts, k = 320, 128, 128, 8, 2
+    norm = _rms_norm(hidden, device)
+    layer = DroplessMoEMLP(
+        hidden, ffn, experts, k, routing=routing, router_normalization=norm, router_scale=True,
+        router_input_scale=hidden**-0.5 * 8, router_per_expert_scale=True, auxiliary_loss_coefficient=0.0,
+        init_std=0.1, dtype=torch.float32, device=device,
+    )  # fmt: skip
+    with torch.no_grad():
+        layer.router_scale.uniform_(0.5, 1.5)
+        layer.router_per_expert_scale.uniform_(0.5, 1.5)
+    layer.train(training)
+    x = torch.randn(tokens, hidden, device=device, requires_grad=True)
+    grad_output = torch.randn(tokens, hidden, device=device)
+    out = layer(x)
+    if training:
+        out.backward(grad_output)
+
+    parameters = (x, layer.router, layer.layer_1, layer.layer_2, norm.weight, layer.router_scale, layer.router_per_expert_scale)
+    leaves = [t.detach().cpu().clone().requires_grad_() for t in parameters]
+    x_cpu, router_weight, weight_1, weight_2, norm_weight, scale, expert_scale = leaves
+
+    def cpu_norm(t):
+        return t * torch.rsqrt((t**2).mean(-1, keepdim=True) + 1e-5) * norm_weight
+
+    router_in = moe_oracle.router_input(x_cpu, cpu_norm, scale, hidden**-0.5 * 8)
+    logits = torch.nn.functional.linear(router_in, router_weight)
+    if routing == "sinkhorn":
+        scores, top_experts = moe_oracle.sinkhorn_routing(logits, k, training)
+    else:
+        routed = moe_oracle.router(logits, k)
+        scores, top_experts = routed.scores, routed.top_experts
+    scores = moe_oracle.per_expert_scale(scores, top_experts, expert_scale)
+    expected = moe_oracle.looped_moe(x_cpu, scores, top_experts, weight_1, weight_2, experts)
+
+    def close(actual, reference, tolerance=2e-4):
+        return (actual.cpu() - reference).abs().max() <= tolerance * reference.abs().max()
+
+    gpu_scores, gpu_experts = layer.route(x.detach())
+    assert torch.equal(gpu_experts.cpu(), top_experts)
+    assert close(gpu_scores.detach(), scores.detach(), 1e-5)
+    assert close(out.detach(), expected.detach())
+    if training:
+        (expected * grad_output.cpu()).sum().backward()
+        assert close(x.grad, x_cpu.grad)
+        for ours, theirs in ((layer.router, router_weight), (norm.weight, norm_weight), (layer.router_scale, scale),
+                             (layer.router_per_expert_scale, expert_scale)):  # fmt: skip
+            assert close(ours.grad, theirs.grad), ours.shape
+        assert close(layer.layer_1.grad_buffer, weight_1.grad) and close(layer.layer_2.grad_buffer, weight_2.grad)
+
+
+def test_sinkhorn_on_the_gpu_matches_the_restatement(device):
+    from fast_llm_amd.functional.routing import sinkhorn, sinkhorn_routing
+
+    generator = torch.Generator().manual_seed(11)
+    logits = torch.randn(500, 16, generator=generator)
+    assert torch.allclose(sinkhorn(logits.to(device)).cpu(), moe_oracle.sinkhorn(logits), rtol=1e-4, atol=1e-9)
+    for k in (1, 3):
+        for training in (True, False):
+            scores, top_experts = sinkhorn_routing(logits.to(device), k, training)
+            expected_scores, expected_experts = moe_oracle.sinkhorn_routing(logits, k, training)
+            assert torch.equal(top_experts.cpu(), expected_experts)
+            assert torch.allclose(scores.cpu(), expected_scores, rtol=1e-5)
+    with pytest.raises(ValueError):
+        from fast_llm_amd.layers.moe import DroplessMoEMLP
+
+        DroplessMoEMLP(64, 64, 4, 1, routing="sinkhorn", shared_experts=1, device=device)

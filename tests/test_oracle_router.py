@@ -93,3 +93,85 @@ def test_router_backward_is_the_derivative_of_the_trained_objective():
             down[t][e] -= step
             numeric = (objective(up) - objective(down)) / (2 * step)
             assert grad[t, e].item() == pytest.approx(numeric, rel=1e-5, abs=1e-8)
+
+
+def test_sinkhorn_balances_rows_and_columns():
+    """What the iteration converges to is fixed by the mathematics: a rescaling d0[t] exp(cost[t, e]) d1[e] whose rows
+    sum to 1 / T exactly after the last row step... and whose columns sum to 1 / E (the last step rescales columns),
+    rows then within the tolerance. The ordering inside a row is changed only through the column scales."""
+    generator = torch.Generator().manual_seed(0)
+    tokens, experts = 96, 8
+    cost = torch.randn(tokens, experts, generator=generator)
+    cost[:, 0] += 2.0  # an expert everybody prefers
+    balanced = moe_oracle.sinkhorn(cost, tolerance=1e-7)
+    assert torch.allclose(balanced.sum(0), torch.full((experts,), 1 / experts), rtol=1e-4)
+    assert torch.allclose(balanced.sum(1), torch.full((tokens,), 1 / tokens), rtol=2e-3)
+    # It is a diagonal rescaling of exp(cost): the ratio to exp(cost) has rank one.
+    ratio = balanced / torch.exp(cost)
+    assert torch.allclose(ratio, ratio[:, :1] * ratio[:1, :] / ratio[0, 0], rtol=1e-4)
+    # Balancing spreads the load: the plain top-1 sends most tokens to expert 0, the balanced one does not.
+    plain = torch.bincount(cost.argmax(-1), minlength=experts)
+    spread = torch.bincount(balanced.argmax(-1), minlength=experts)
+    assert plain[0] > tokens // 2 and spread.max() <= 2 * tokens // experts
+
+
+def test_sinkhorn_against_a_python_loop():
+    generator = torch.Generator().manual_seed(1)
+    tokens, experts, tolerance, eps = 5, 3, 1e-5, 1e-9
+    cost = torch.randn(tokens, experts, generator=generator)
+    c = [[math.exp(v) for v in row] for row in cost.tolist()]
+    d0, d1 = [1.0] * tokens, [1.0] * experts
+    while True:
+        d0 = [(1 / tokens) / (sum(d1[e] * c[t][e] for e in range(experts)) + eps) for t in range(tokens)]
+        new = [(1 / experts) / (sum(d0[t] * c[t][e] for t in range(tokens)) + eps) for e in range(experts)]
+        error = sum(abs(a - b) for a, b in zip(new, d1)) / experts
+        d1 = new
+        if not error > tolerance:
+            break
+    expected = torch.tensor([[d0[t] * c[t][e] * d1[e] for e in range(experts)] for t in range(tokens)])
+    assert torch.allclose(moe_oracle.sinkhorn(cost, tolerance, eps), expected, rtol=1e-5)
+
+
+@pytest.mark.parametrize("k", [1, 2])
+def test_sinkhorn_routing_scores_are_the_activated_logits(k):
+    generator = torch.Generator().manual_seed(2)
+    logits = torch.randn(40, 6, generator=generator)
+    for training in (True, False):
+        scores, top_experts = moe_oracle.sinkhorn_routing(logits, k, training)
+        for t in range(logits.size(0)):
+            row = logits[t].tolist()
+            if k == 1:
+                activated = [1 / (1 + math.exp(-v)) for v in row]
+            else:
+                total = sum(math.exp(v) for v in row)
+                activated = [math.exp(v) / total for v in row]
+            for j in range(k):
+                assert scores[t, j].item() == pytest.approx(activated[top_experts[t, j]], rel=1e-5)
+            if not training:  # plain top-k of the activated logits, in descending order
+                order = sorted(range(len(row)), key=lambda e: -row[e])[:k]
+                assert top_experts[t].tolist() == order
+        assert len({tuple(sorted(r)) for r in top_experts.tolist()}) > 1
+
+
+def test_router_input_and_per_expert_scale():
+    generator = torch.Generator().manual_seed(3)
+    x = torch.randn(7, 5, generator=generator)
+    scale = torch.rand(5, generator=generator) + 0.5
+
+    def rms(t):
+        return t / torch.sqrt((t * t).mean(-1, keepdim=True) + 1e-5)
+
+    out = moe_oracle.router_input(x, rms, scale, 5**-0.5)
+    for t in range(7):
+        row = x[t].tolist()
+        norm = math.sqrt(sum(v * v for v in row) / 5 + 1e-5)
+        for h in range(5):
+            assert out[t, h].item() == pytest.approx(row[h] / norm * scale[h].item() * 5**-0.5, rel=1e-5)
+    assert moe_oracle.router_input(x) is x
+    scores, top = torch.rand(7, 2, generator=generator), torch.randint(0, 4, (7, 2), generator=generator)
+    per_expert = torch.tensor([1.0, 2.0, 0.5, 3.0])
+    scaled = moe_oracle.per_expert_scale(scores, top, per_expert)
+    for t in range(7):
+        for j in range(2):
+            assert scaled[t, j].item() == pytest.approx(scores[t, j].item() * per_expert[top[t, j]].item())
+    assert moe_oracle.per_expert_scale(scores, top, None) is scores
