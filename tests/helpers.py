@@ -23,6 +23,32 @@ def max_rel_err(x: torch.Tensor, y: torch.Tensor) -> float:
     return diff / scale if scale > 0 else diff
 
 
+def rel_rms_err(x: torch.Tensor, y: torch.Tensor) -> float:
+    """||x - y|| / ||y||: the relative RMS error of the reference's benchmark runner
+    (tools/benchmark/triton_kernels/runner.py:305-312)."""
+    scale = torch.norm(y.double(), 2).item()
+    diff = torch.norm(x.double() - y.double(), 2).item()
+    return diff / scale if scale > 0 else diff
+
+
+def max_block_rel_err(x: torch.Tensor, y: torch.Tensor, block_rows: int = 256, block_columns: int = 256) -> float:
+    """max over blocks (the size of a kernel tile) of max|x - y| in the block / max|y| in the block: a wrong tile of
+    small values cannot hide behind a large value elsewhere in the tensor. A block where y is all zero counts its
+    absolute error. Runs on the tensors' device."""
+    assert x.shape == y.shape and x.dim() == 2
+    rows, columns = x.shape
+    padded_rows, padded_columns = -(-rows // block_rows) * block_rows, -(-columns // block_columns) * block_columns
+
+    def block_max(t: torch.Tensor) -> torch.Tensor:
+        padded = torch.zeros(padded_rows, padded_columns, dtype=torch.float32, device=t.device)
+        padded[:rows, :columns] = t
+        return padded.view(padded_rows // block_rows, block_rows, padded_columns // block_columns, block_columns).amax(dim=(1, 3))
+
+    diff = block_max((x.float() - y.float()).abs())
+    scale = block_max(y.float().abs())
+    return torch.where(scale > 0, diff / scale.clamp_min(1e-30), diff).max().item()
+
+
 def fixture_sparse_map(case: dict, dtype: torch.dtype = torch.int64) -> moe_oracle.OracleSparseMap:
     """The hand-built map of the reference's sparse-matmul tests (tests/functional/test_sparse_matmul.py:51-62):
     only expert_ends, expert_pad_begins, num_rows and num_experts are set."""

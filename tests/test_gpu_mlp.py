@@ -10,7 +10,7 @@ from fast_llm_amd.functional.sparse_copy import get_sparse_map
 from fast_llm_amd.layers.moe import DroplessMoEMLP, attach_grad_buffer
 from fast_llm_amd.workloads import WORKLOADS, MoEWorkload, make_inputs
 from oracle import moe_oracle
-from tests.helpers import REFERENCE_FIXTURES, max_rel_err, rms_diff
+from tests.helpers import REFERENCE_FIXTURES, max_block_rel_err, max_rel_err, rel_rms_err, rms_diff
 
 pytestmark = pytest.mark.gpu
 
@@ -204,9 +204,21 @@ def test_benchmark_configurations_full_size(name, device):
         workload.experts, gpu.grad_output.float(),
     )
     for name_, ours in zip(_NAMES, actual):
+        theirs = getattr(expected, name_)
         assert torch.isfinite(ours).all(), name_
-        error = max_rel_err(ours, getattr(expected, name_))
+        error = max_rel_err(ours, theirs)
         assert error <= 1e-2, f"{name_}: {error}"
+        # The reference's own metric, relative RMS (tools/benchmark/triton_kernels/runner.py:305-312): bf16 rounds
+        # every stored intermediate to 2^-9 relative, so a correct result sits at a few 1e-3.
+        error = rel_rms_err(ours, theirs)
+        assert error <= 1e-2, f"{name_}: relative rms {error}"
+        # Tile by tile (256 x 256, the grouped products' tile; 128 rows for the token-major tensors, the padding unit):
+        # the error of every block against that block's own largest value. bf16 rounding stays below 2e-2 there; a
+        # block computed from the wrong operands is off by order 1.
+        if ours.dim() == 2 and ours.size(1) >= 256:
+            block_rows = 256 if name_.startswith("grad_weight") else 128
+            error = max_block_rel_err(ours, theirs, block_rows, 256)
+            assert error <= 2e-2, f"{name_}: worst block {error}"
     counts = torch.bincount(inputs.top_experts.flatten(), minlength=workload.experts)
     if name.startswith("imbalanced"):
         assert counts.max() > 2.5 * counts.float().mean()
@@ -255,7 +267,8 @@ def test_dynamic_shape_and_micro_batches_accumulate(device):
 @pytest.mark.parametrize("activation", ["silu", "gelu", "relu", "squared_relu", "identity"])
 def test_fused_activation_epilogues_are_bit_identical(activation, recompute_level, device, monkeypatch):
     """The gated activation inside the grouped products' epilogues (forward in layer 1, backward in the layer 2
-    input gradient) against the separate kernels: every output and gradient, bit for bit, ragged experts included."""
+    input gradient): every output and gradient against the oracle's dropless MLP at this shape, and bit for bit
+    against the separate kernels, ragged experts included."""
     from fast_llm_amd import _lib
     from fast_llm_amd.functional.config import KernelConfig
 
@@ -273,6 +286,14 @@ def test_fused_activation_epilogues_are_bit_identical(activation, recompute_leve
         assert any(label.startswith("fm_mlp_activation") for label in labels) == (not fused)
     for fused, separate in zip(results[True], results[False]):
         assert torch.equal(fused, separate)
+    oracle_map = moe_oracle.sparse_map(inputs.top_experts, workload.experts)
+    expected = moe_oracle.dropless_mlp_forward_backward(
+        inputs.hidden_states, inputs.scores, inputs.weight_1, inputs.weight_2, oracle_map, inputs.grad_output,
+        activation=activation,
+    )  # fmt: skip
+    for name, ours in zip(_NAMES, results[True]):
+        assert max_rel_err(ours.cpu(), getattr(expected, name)) <= 1e-2, name
+        assert rel_rms_err(ours.cpu(), getattr(expected, name)) <= 1e-2, name
 
 
 def test_step_replays_from_a_hip_graph(device):
