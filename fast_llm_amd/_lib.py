@@ -7,6 +7,7 @@ raises. Build it with `python -m fast_llm_amd.build`.
 
 import ctypes
 import pathlib
+import warnings
 
 import torch
 
@@ -56,6 +57,7 @@ SIGNATURES: dict[str, tuple] = {
 }
 
 FM_ERR_INVALID_ARGUMENT, FM_ERR_UNSUPPORTED, FM_ERR_LAUNCH = -1, -2, -3
+FM_NOTE_GENERIC_KERNEL = 1
 
 DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 INDEX_DTYPES = {torch.int16: 0, torch.int32: 1, torch.int64: 2}
@@ -97,8 +99,17 @@ def lib() -> ctypes.CDLL:
 
 
 def check(status: int) -> None:
-    """Turn a negative `fm_status` into the exception the reference's Python code would raise."""
+    """Turn a negative `fm_status` into the exception the reference's Python code would raise; a positive one (the
+    call went through, with a remark) into a warning."""
     if status == 0:
+        return
+    if status == FM_NOTE_GENERIC_KERNEL:
+        warnings.warn(
+            "a grouped product with half-precision operands ran on the generic multiply-add kernel, not on the matrix "
+            "cores (operands need a unit stride on one axis, 16-byte aligned rows, a reduction that is a multiple of 64)",
+            RuntimeWarning,
+            stacklevel=3,
+        )
         return
     message = lib().fm_last_error().decode()
     if status == FM_ERR_LAUNCH:

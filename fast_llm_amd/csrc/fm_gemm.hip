@@ -10,18 +10,19 @@
 // Half-precision operands with vectorisable layouts go to the MFMA kernel (fm_gemm_mfma.hip). Everything else
 // (fp32 operands, odd strides or sizes) goes to the generic kernel below: a 64 x 64 x 16 LDS-tiled kernel with
 // full bounds checks and true fp32 multiply-adds, which is also what the 1e-5 fp32 parity bound needs. The
-// generic kernel takes the expert of a 64-row block from its first row, so there expert boundaries must be
-// multiples of 64 rows.
+// generic kernel computes a 64-row block that straddles an expert boundary in one pass per expert, so it takes any
+// padding multiple.
 #include "fm_gemm_common.h"
 
 namespace fm {
 
-// Where one output tile of the generic kernel reads and writes. Offsets are in elements.
+// Where one output tile (or the part of it that belongs to one expert) reads and writes. Offsets are in elements.
 struct TileWork {
     int64_t lhs_offset;  // element (first row of tile, k = 0)
     int64_t rhs_offset;  // element (k = 0, first column of tile)
     int64_t out_offset;
     int64_t k_lo, k_hi;  // valid reduction range; outside it operands count as zero
+    int row_lo, row_hi;  // rows of the tile, relative to its first row, that this piece of work covers
     bool skip;
 };
 
@@ -36,11 +37,18 @@ __device__ __forceinline__ int expert_of_row(const GemmArgs &args, int64_t row) 
     return lo;
 }
 
-__device__ __forceinline__ TileWork resolve_tile(const GemmArgs &args, int64_t row0, int64_t col0) {
+constexpr int kGenTile = 64, kGenK = 16, kGenThreads = 256;
+
+// The work of the tile at (row0, col0) for the expert that owns its row `first_row` (relative to row0): in the
+// products whose rows are grouped by expert, a tile that straddles an expert boundary (any padding multiple is
+// allowed) is computed in one piece per expert.
+__device__ __forceinline__ TileWork resolve_tile(const GemmArgs &args, int64_t row0, int64_t col0, int first_row) {
     TileWork work;
     work.skip = false;
     work.k_lo = 0;
     work.k_hi = args.inner;
+    work.row_lo = first_row;
+    work.row_hi = kGenTile;
     work.out_offset = row0 * args.out_stride_row + col0 * args.out_stride_col;
     const bool dense = args.expert_ends == nullptr;
     if (args.mode == kInputRowSparse) {
@@ -55,10 +63,14 @@ __device__ __forceinline__ TileWork resolve_tile(const GemmArgs &args, int64_t r
             if (work.k_lo < 0) work.k_lo = 0;
         }
     } else {
-        const int expert = dense ? 0 : expert_of_row(args, row0);
+        const int expert = dense ? 0 : expert_of_row(args, row0 + first_row);
         if (expert >= args.num_experts) {
             work.skip = true;  // phantom rows past the last expert
             return work;
+        }
+        if (!dense) {
+            const int64_t end = load_index(args.expert_ends, args.index_dtype, expert);
+            if (end - row0 < work.row_hi) work.row_hi = static_cast<int>(end - row0);
         }
         work.lhs_offset = row0 * args.lhs_stride_row;
         if (args.mode == kOutputSparse)
@@ -73,77 +85,81 @@ __device__ __forceinline__ TileWork resolve_tile(const GemmArgs &args, int64_t r
 // =========================================================================================================
 // Generic path
 // =========================================================================================================
-constexpr int kGenTile = 64, kGenK = 16, kGenThreads = 256;
-
 template <typename T>
 __global__ __launch_bounds__(kGenThreads) void grouped_gemm_generic_kernel(GemmArgs args) {
     __shared__ float lds_a[kGenK][kGenTile + 1];
     __shared__ float lds_b[kGenK][kGenTile + 1];
     const int tile_n = blockIdx.x % args.tiles_n, tile_m = blockIdx.x / args.tiles_n;
     const int64_t row0 = static_cast<int64_t>(tile_m) * kGenTile, col0 = static_cast<int64_t>(tile_n) * kGenTile;
-    const TileWork work = resolve_tile(args, row0, col0);
-    if (work.skip) return;
-
-    const T *lhs = static_cast<const T *>(args.lhs) + work.lhs_offset;
-    const T *rhs = static_cast<const T *>(args.rhs) + work.rhs_offset;
     // Rows/columns of this tile that exist (a row-sparse tile must also stay inside its expert's block of out).
     int64_t rows_here = args.rows - row0, cols_here = args.cols - col0;
     if (args.mode == kInputRowSparse) {
         const int64_t left_in_expert = args.sparse_size - row0 % args.sparse_size;
         if (left_in_expert < rows_here) rows_here = left_in_expert;
     }
+    if (rows_here > kGenTile) rows_here = kGenTile;
     const int thread_m = threadIdx.x / 16, thread_n = threadIdx.x % 16;
-    float acc[4][4] = {};
 
-    for (int64_t k0 = work.k_lo / kGenK * kGenK; k0 < work.k_hi; k0 += kGenK) {
-        for (int i = threadIdx.x; i < kGenK * kGenTile; i += kGenThreads) {
-            // lhs: consecutive threads along the axis with the smaller stride
-            int k_local, r_local;
-            if (args.lhs_stride_inner <= args.lhs_stride_row) { k_local = i % kGenK; r_local = i / kGenK; }
-            else { r_local = i % kGenTile; k_local = i / kGenTile; }
-            int64_t k = k0 + k_local;
-            float value = 0.f;
-            if (r_local < rows_here && k >= work.k_lo && k < work.k_hi)
-                value = to_float(lhs[r_local * args.lhs_stride_row + k * args.lhs_stride_inner]);
-            lds_a[k_local][r_local] = value;
+    // One pass per expert that owns rows of the tile (a single pass unless the tile straddles a boundary).
+    for (int first_row = 0; first_row < rows_here;) {
+        const TileWork work = resolve_tile(args, row0, col0, first_row);
+        if (work.skip) return;  // the rest of the tile lies past the last expert
+        const int row_hi = work.row_hi < rows_here ? work.row_hi : static_cast<int>(rows_here);
+        const T *lhs = static_cast<const T *>(args.lhs) + work.lhs_offset;
+        const T *rhs = static_cast<const T *>(args.rhs) + work.rhs_offset;
+        float acc[4][4] = {};
 
-            int c_local;
-            if (args.rhs_stride_inner <= args.rhs_stride_col) { k_local = i % kGenK; c_local = i / kGenK; }
-            else { c_local = i % kGenTile; k_local = i / kGenTile; }
-            k = k0 + k_local;
-            value = 0.f;
-            if (c_local < cols_here && k >= work.k_lo && k < work.k_hi)
-                value = to_float(rhs[k * args.rhs_stride_inner + c_local * args.rhs_stride_col]);
-            lds_b[k_local][c_local] = value;
+        for (int64_t k0 = work.k_lo / kGenK * kGenK; k0 < work.k_hi; k0 += kGenK) {
+            for (int i = threadIdx.x; i < kGenK * kGenTile; i += kGenThreads) {
+                // lhs: consecutive threads along the axis with the smaller stride
+                int k_local, r_local;
+                if (args.lhs_stride_inner <= args.lhs_stride_row) { k_local = i % kGenK; r_local = i / kGenK; }
+                else { r_local = i % kGenTile; k_local = i / kGenTile; }
+                int64_t k = k0 + k_local;
+                float value = 0.f;
+                if (r_local >= first_row && r_local < row_hi && k >= work.k_lo && k < work.k_hi)
+                    value = to_float(lhs[r_local * args.lhs_stride_row + k * args.lhs_stride_inner]);
+                lds_a[k_local][r_local] = value;
+
+                int c_local;
+                if (args.rhs_stride_inner <= args.rhs_stride_col) { k_local = i % kGenK; c_local = i / kGenK; }
+                else { c_local = i % kGenTile; k_local = i / kGenTile; }
+                k = k0 + k_local;
+                value = 0.f;
+                if (c_local < cols_here && k >= work.k_lo && k < work.k_hi)
+                    value = to_float(rhs[k * args.rhs_stride_inner + c_local * args.rhs_stride_col]);
+                lds_b[k_local][c_local] = value;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < kGenK; ++k) {
+                float a[4], b[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[i] = lds_a[k][thread_m + 16 * i];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) b[j] = lds_b[k][thread_n + 16 * j];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+            }
+            __syncthreads();
         }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < kGenK; ++k) {
-            float a[4], b[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = lds_a[k][thread_m + 16 * i];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = lds_b[k][thread_n + 16 * j];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
-        }
-        __syncthreads();
-    }
 
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = thread_m + 16 * i;
-        if (row >= rows_here) continue;
+        for (int i = 0; i < 4; ++i) {
+            const int row = thread_m + 16 * i;
+            if (row < first_row || row >= row_hi) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int column = thread_n + 16 * j;
-            if (column >= cols_here) continue;
-            store_out_dyn(args.out, args.out_dtype,
-                          work.out_offset + row * args.out_stride_row + column * args.out_stride_col, acc[i][j],
-                          args.accumulate != 0);
+            for (int j = 0; j < 4; ++j) {
+                const int column = thread_n + 16 * j;
+                if (column >= cols_here) continue;
+                store_out_dyn(args.out, args.out_dtype,
+                              work.out_offset + row * args.out_stride_row + column * args.out_stride_col, acc[i][j],
+                              args.accumulate != 0);
+            }
         }
+        first_row = row_hi;
     }
 }
 
@@ -162,9 +178,12 @@ static int run_gemm(const char *name, GemmArgs args, int dtype, void *workspace,
     FM_REQUIRE(args.out && (args.inner == 0 || (args.lhs && args.rhs)), "%s: null tensor", name);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
 
+    int note = FM_OK;
     if (mfma_gemm_eligible(args, dtype)) {
         if (int status = mfma_gemm_launch(args, dtype, workspace, workspace_size, stream)) return status;
     } else {
+        // Half-precision operands that the matrix-core kernel cannot take: correct, but far slower. Say so.
+        if (dtype != FM_DTYPE_F32) note = FM_NOTE_GENERIC_KERNEL;
         // A row-sparse tile must not cross into the next expert's block of out.
         if (args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % kGenTile != 0)
             return fail(FM_ERR_UNSUPPORTED, "%s: row_sparse_dim=%lld must be a multiple of %d", name,
@@ -175,7 +194,8 @@ static int run_gemm(const char *name, GemmArgs args, int dtype, void *workspace,
         const int grid = args.tiles_m * args.tiles_n;
         FM_DISPATCH_DTYPE(dtype, T, { grouped_gemm_generic_kernel<T><<<grid, kGenThreads, 0, stream>>>(args); });
     }
-    return check_launch(name);
+    if (int status = check_launch(name)) return status;
+    return note;
 }
 
 }  // namespace fm

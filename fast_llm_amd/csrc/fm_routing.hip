@@ -20,9 +20,13 @@ struct Candidate {
     int index;
 };
 
-// The larger value wins; equal values: the lower index. NaN never wins against a number.
+// The larger value wins; equal values: the lower index. NaN counts as larger than every number, as in torch.topk
+// (the reference's routing, fast_llm/layers/decoder/mlp/mixture_of_experts.py:243): a token with a NaN logit selects
+// that expert and gets NaN scores, so a broken router shows in the loss instead of silently losing a slot.
 __device__ __forceinline__ Candidate better(Candidate a, Candidate b) {
-    const bool take_b = b.value > a.value || (b.value == a.value && b.index < a.index) || (a.value != a.value && b.value == b.value);
+    const bool a_nan = a.value != a.value, b_nan = b.value != b.value;
+    const bool same = a_nan == b_nan && (a_nan || a.value == b.value);
+    const bool take_b = (b_nan && !a_nan) || (!a_nan && !b_nan && b.value > a.value) || (same && b.index < a.index);
     return take_b ? b : a;
 }
 

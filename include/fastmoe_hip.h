@@ -7,8 +7,8 @@
  *     stream) and never synchronises, allocates or frees device memory, or keeps a caller's pointer after it
  *     returns: outputs and every workspace are the caller's, and a workspace may be reused as soon as the stream
  *     has passed the call;
- *   - returns `FM_OK` (0) or a negative `fm_status`; the message for the calling thread is read with
- *     `fm_last_error()`. No C++ exception crosses this boundary.
+ *   - returns `FM_OK` (0), a positive remark (the work was launched), or a negative `fm_status`; the message of a
+ *     negative status for the calling thread is read with `fm_last_error()`. No C++ exception crosses this boundary.
  *
  * The reference (ServiceNow/Fast-LLM) has no FFI for this path: its "operator API" is a set of Python
  * callables that launch Triton kernels. Each function below replaces the kernel launch inside one of those
@@ -36,6 +36,10 @@ enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
 enum fm_index_dtype { FM_INDEX_I16 = 0, FM_INDEX_I32 = 1, FM_INDEX_I64 = 2 };
 
 enum fm_status {
+    /* Positive: the call succeeded and was launched, with a remark. The three grouped products return this one when
+     * bf16/fp16 operands had to take the bounds-checked multiply-add kernel instead of the matrix cores (a stride
+     * that is not 1 on either axis, rows not 16-byte aligned, reduction not a multiple of 64, stride >= 2^21). */
+    FM_NOTE_GENERIC_KERNEL = 1,
     FM_OK = 0,
     FM_ERR_INVALID_ARGUMENT = -1, /* bad enum, negative size, null pointer, misaligned/unsupported stride */
     FM_ERR_UNSUPPORTED = -2,      /* valid request that this build has no kernel for */
@@ -231,7 +235,8 @@ int fm_mlp_activation_backward(const void *grad_output, void *grad_input, const 
  * content of `out` is added (in fp32) before the store. `expert_ends` (and `expert_pad_begins`) have
  * `index_dtype`; the expert of a 128-row block is `#{e : expert_ends[e] <= first row of the block}`, so every
  * expert boundary must be a multiple of 128 rows (the reference's MAX_DROPLESS_BLOCK_SIZE_ROW contract,
- * fast_llm/functional/config.py:106, sparse_linear.py:274). If `expert_ends` is NULL the product is an
+ * fast_llm/functional/config.py:106, sparse_linear.py:274; the kernels here take any boundary: a multiple of 128 is
+ * only what keeps the matrix-core tiles full). If `expert_ends` is NULL the product is an
  * ordinary dense one (a single expert owning all rows), which is what the reference does for
  * `sparse_map=None` (sparse_linear.py:276-277, 404-405, 537-538).
  * Results are deterministic (no floating-point atomics; every sum has a fixed order that depends only on the

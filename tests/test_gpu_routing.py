@@ -363,3 +363,25 @@ def test_sinkhorn_on_the_gpu_matches_the_restatement(device):
         from fast_llm_amd.layers.moe import DroplessMoEMLP
 
         DroplessMoEMLP(64, 64, 4, 1, routing="sinkhorn", shared_experts=1, device=device)
+
+
+def test_nan_logits_rank_highest_like_torch_topk(device):
+    """A NaN logit is selected first (torch.topk's order, which the reference's routing inherits) and makes the
+    token's scores NaN; every slot still names a valid expert, and other tokens are unaffected. Both routing kernels."""
+    generator = torch.Generator().manual_seed(5)
+    logits = torch.randn(64, 8, generator=generator)
+    logits[3, 6] = float("nan")
+    logits[10, 0] = logits[10, 7] = float("nan")  # two NaNs: the lower expert first
+    expected_scores, expected_experts = moe_oracle.topk_routing(logits, 2)
+    for function in (
+        lambda: topk_routing(logits.to(device), 2),
+        lambda: router(logits.to(device), 2)[:2],
+    ):
+        scores, top_experts = function()
+        assert top_experts[3, 0].item() == 6 and top_experts[10].tolist() == [0, 7]
+        assert ((top_experts >= 0) & (top_experts < 8)).all()
+        clean = torch.ones(64, dtype=torch.bool)
+        clean[[3, 10]] = False
+        assert torch.equal(top_experts.cpu()[clean], expected_experts[clean])
+        assert torch.allclose(scores.cpu()[clean], expected_scores[clean], rtol=2e-6, atol=1e-7)
+        assert torch.isnan(scores[3]).all() and torch.isnan(scores[10]).all()

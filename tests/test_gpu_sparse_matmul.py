@@ -458,3 +458,55 @@ def test_random_shapes_through_the_matrix_core_kernel(seed, device):
     input_row_sparse_matmul(x_gpu.t(), y.to(device), sparse_map, out=out)
     expected = moe_oracle.input_row_sparse_matmul(x.t(), y, oracle_map, out=torch.zeros(out.shape, dtype=out_dtype))
     assert max_rel_err(out.cpu(), expected) <= tolerance
+
+
+@pytest.mark.parametrize("pad", [32, 8, 1])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_expert_boundaries_inside_a_tile(pad, dtype, device):
+    """Expert blocks padded to less than a kernel tile (`get_sparse_map(pad_to_multiple=...)` allows any multiple):
+    tiles that straddle expert boundaries are computed expert by expert, in the fp32 multiply-add kernel (64-row
+    blocks) and in the matrix-core kernel (tiles enumerated per expert) alike."""
+    experts, inner, other = 7, 64, 72
+    case = _ragged_case(pad, experts, pad=pad)
+    oracle_map = fixture_sparse_map(case)
+    oracle_map.num_rows = case["expert_ends"][-1] + case["phantom_rows"]
+    assert any(end % 64 for end in case["expert_ends"])
+    sparse_map = to_device_map(oracle_map, device, torch.int32)
+    used = _used_rows(oracle_map)
+    generator = torch.Generator().manual_seed(17)
+    x = _normal(oracle_map.num_rows, inner, dtype, generator)
+    x[~oracle_map.real_row_mask()] = 0
+    weight = _normal(experts * other, inner, dtype, generator)
+    tolerance = _MAX_REL[dtype]
+
+    out = torch.full((oracle_map.num_rows, other), 5.0, dtype=dtype, device=device)
+    output_sparse_matmul(x.to(device), weight.to(device).t(), sparse_map, out)
+    expected = moe_oracle.output_sparse_matmul(x, weight.t(), oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+    assert (out[used:] == 5.0).all()
+
+    weight_inner = _normal(experts * inner, other, dtype, generator)
+    out = input_inner_sparse_matmul(x.to(device), weight_inner.to(device), sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(x, weight_inner, oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= tolerance
+
+    y = _normal(oracle_map.num_rows, other, dtype, generator)
+    out = input_row_sparse_matmul(x.to(device).t(), y.to(device), sparse_map)
+    expected = moe_oracle.input_row_sparse_matmul(x.t(), y, oracle_map)
+    assert max_rel_err(out.cpu(), expected) <= tolerance
+
+
+def test_half_precision_on_the_generic_kernel_warns(device):
+    """bf16 operands the matrix-core kernel cannot take (here: a reduction that is not a multiple of 64) still give the
+    right product, from the multiply-add kernel, and the wrapper says so."""
+    generator = torch.Generator().manual_seed(19)
+    lhs, rhs = _normal(130, 100, torch.bfloat16, generator), _normal(100, 72, torch.bfloat16, generator)
+    with pytest.warns(RuntimeWarning, match="generic multiply-add kernel"):
+        out = dense_matmul(lhs.to(device), rhs.to(device))
+    assert max_rel_err(out.cpu(), (lhs.float() @ rhs.float()).to(torch.bfloat16)) <= 1e-2
+    import warnings
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        dense_matmul(_normal(128, 128, torch.bfloat16, generator).to(device), _normal(128, 72, torch.bfloat16, generator).to(device))
+        dense_matmul(lhs.float().to(device), rhs.float().to(device))  # fp32 belongs on that kernel: no remark

@@ -175,3 +175,12 @@ def test_router_input_and_per_expert_scale():
         for j in range(2):
             assert scaled[t, j].item() == pytest.approx(scores[t, j].item() * per_expert[top[t, j]].item())
     assert moe_oracle.per_expert_scale(scores, top, None) is scores
+
+
+def test_nan_logits_rank_highest_like_torch_topk():
+    """The contract for a NaN router logit is torch.topk's (the reference routes with it): NaN ranks above every
+    number, the token selects that expert, and its scores are NaN."""
+    logits = torch.tensor([[0.5, float("nan"), 2.0, 1.0], [3.0, 1.0, 2.0, 0.0]])
+    scores, top_experts = moe_oracle.topk_routing(logits, 2)
+    assert top_experts[0].tolist() == [1, 2] and top_experts[1].tolist() == [0, 2]
+    assert torch.isnan(scores[0]).all() and torch.isfinite(scores[1]).all()
