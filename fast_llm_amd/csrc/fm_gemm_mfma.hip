@@ -525,16 +525,18 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int
 // 16-byte write, and the staged rows are read back as 16-byte chunks in row-major order, all reads of a 32-row block
 // before the first store, so that a store instruction covers full 256-byte row segments.
 // `source(i)` yields the wavefront's accumulators of its i-th block of 32 rows, as something indexed [j][register].
+// `row_base`: first tile row of this wavefront; `blocks`: how many 32-row blocks it holds (4, or 2 in a half tile).
 template <typename OutT, bool kAccumulate, typename Source>
 __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, OutT *out, int64_t stride,
-                                           int rows_valid, int cols_valid, int wave, int lane) {
+                                           int rows_valid, int cols_valid, int wave, int lane, int row_base,
+                                           int blocks) {
     using StageT = std::conditional_t<kAccumulate, float, OutT>;
     constexpr int kChunk = 16 / sizeof(StageT);         // elements per 16-byte chunk
     constexpr int kLanesPerRow = kWaveCols / kChunk;    // 16 or 32
     constexpr int kRowsPerRead = 64 / kLanesPerRow;     // 4 or 2
     constexpr int kReads = 32 / kRowsPerRead;           // 8 or 16
     constexpr int kRowBytes = kWaveCols * sizeof(StageT) + kEpiloguePadBytes;
-    const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
+    const int wave_n = wave % kWavesN;
     FM_LDS(char) *staging = lds + wave * (32 * kRowBytes);
     FM_LDS(char) *write_base = staging + (lane & 31) * kRowBytes + (lane >> 5) * 4 * sizeof(StageT);
     const int read_row = lane / kLanesPerRow, read_column = (lane % kLanesPerRow) * kChunk;
@@ -542,7 +544,7 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
     const int column_in_tile = wave_n * kWaveCols + read_column;
     // cols_valid is a multiple of 8, so a chunk of 4 or 8 columns is valid or not as a whole.
     const bool column_ok = column_in_tile < cols_valid;
-    const int first_row = wave_m * kWaveRows + read_row;
+    const int first_row = row_base + read_row;
     OutT *pointer = out + first_row * stride + column_in_tile;
     const bool whole_tile = rows_valid == kTile && cols_valid == kTile;
     constexpr bool kAhead = sizeof(OutT) == 2;
@@ -556,6 +558,7 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
     };
 #pragma unroll
     for (int i = 0; i < kTilesM; ++i) {
+        if (i >= blocks) break;  // wave-uniform
         auto &&block = source(i);
         // When adding to `out`: what it holds is requested ahead of time, all chunks of a row block at once and one
         // block ahead of the block being staged, so that the loads are on their way while accumulators go through
@@ -564,7 +567,7 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
         // (One block ahead only where the values are two bytes wide: two blocks of fp32 do not fit the registers.)
         if constexpr (kAccumulate && kAhead) {
             if (i == 0) load_previous(0, previous[0]);
-            if (i + 1 < kTilesM) load_previous(i + 1, previous[(i + 1) & 1]);
+            if (i + 1 < blocks) load_previous(i + 1, previous[(i + 1) & 1]);
         } else if constexpr (kAccumulate) {
             load_previous(i, previous[0]);
         }
@@ -756,17 +759,17 @@ __device__ __forceinline__ void store_tile_gated_forward(const f32x16_t (&acc)[k
 
 template <typename Source>
 __device__ __forceinline__ void store_result(const GemmArgs &args, const TileWork &work, Source &&source,
-                                             FM_LDS(char) * lds, int wave, int lane) {
+                                             FM_LDS(char) * lds, int wave, int lane, int row_base, int blocks) {
     const bool accumulate = args.accumulate != 0;
     auto store = [&](auto *out) {
         if (accumulate)
             store_tile<std::remove_pointer_t<decltype(out)>, true>(source, lds, out + work.out_offset,
                                                                    args.out_stride_row, work.rows_valid,
-                                                                   work.cols_valid, wave, lane);
+                                                                   work.cols_valid, wave, lane, row_base, blocks);
         else
             store_tile<std::remove_pointer_t<decltype(out)>, false>(source, lds, out + work.out_offset,
                                                                     args.out_stride_row, work.rows_valid,
-                                                                    work.cols_valid, wave, lane);
+                                                                    work.cols_valid, wave, lane, row_base, blocks);
     };
     if (args.out_dtype == FM_DTYPE_F32) store(static_cast<float *>(args.out));
     else if (args.out_dtype == FM_DTYPE_BF16) store(static_cast<bf16_t *>(args.out));
@@ -824,6 +827,12 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     const int64_t k_first = work.k_lo / kBK * kBK;
     const int64_t k_last = work.k_hi > work.k_lo ? (work.k_hi + kBK - 1) / kBK * kBK : k_first;
     const int num_slices = __builtin_amdgcn_readfirstlane(static_cast<int>((k_last - k_first) / kBK));
+    // A tile with at most 128 valid rows (the last row tile of an expert whose padded row count is an odd multiple of
+    // 128) is a half tile: the wavefronts share its 128 rows, 64 each, and issue half the MFMAs. The transfers stay as
+    // they are (the rows past the valid ones bring zeros or repeats that nobody reads).
+    const bool half_tile = kFusion == kFusionNone && piece_slot < 0 && work.rows_valid <= kTile / 2;  // wave-uniform
+    const int wave_row_base = wave_m * (half_tile ? kWaveRows / 2 : kWaveRows);
+    const int wave_row_blocks = half_tile ? kTilesM / 2 : kTilesM;
 
     TileLoader<kLhsContiguousK> load_lhs;
     TileLoader<kRhsContiguousK> load_rhs;
@@ -870,7 +879,7 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     int lhs_frag0[4], lhs_frag[4], lhs_frag_next[4], rhs_frag[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        lhs_frag0[q] = fragment_base<kLhsContiguousK>(wave_m * kWaveRows, q, lane);
+        lhs_frag0[q] = fragment_base<kLhsContiguousK>(wave_row_base, q, lane);
         lhs_frag[q] = lhs_frag0[q] + lhs_now;
         lhs_frag_next[q] = lhs_frag0[q] + lhs_next;
         rhs_frag[q] = fragment_base<kRhsContiguousK>(wave_n * kWaveCols, q, lane);
@@ -899,9 +908,13 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     //   slots 4..7     lhs fragments 0..3 of the next K-step
     //   slots 8..11    in K-steps 0 and 3: four rhs loads
     //   slots 12, 13   two lhs loads
+    // A half tile has 8 slots per K-step (2 x 4 accumulators): rhs fragments in slots 0..3, the two lhs fragments in
+    // slots 4, 5, the rhs loads in slots 2..5 as well and the lhs loads in slots 6, 7.
     static_assert(kTilesM == 4 && kTilesN == 4 && kLoadsPerOperand == 8, "the slot table below is written for this shape");
-    auto iteration = [&](int t, auto slot_constant) {
+    auto iteration = [&](int t, auto slot_constant, auto half_constant) {
         constexpr int kSlot = decltype(slot_constant)::value, kNextSlot = 1 - kSlot;  // rhs, of slices t, t + 1
+        constexpr bool kHalf = decltype(half_constant)::value;
+        constexpr int kRowBlocks = kHalf ? kTilesM / 2 : kTilesM;
 #pragma unroll
         for (int kstep = 0; kstep < kSteps; ++kstep) {
             const bool last = kstep + 1 == kSteps;
@@ -914,11 +927,20 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
                 load_rhs.advance();
             }
 #pragma unroll
-            for (int m = 0; m < kTilesM * kTilesN; ++m) {
+            for (int m = 0; m < kRowBlocks * kTilesN; ++m) {
                 // Boustrophedon order: consecutive MFMAs always share one operand (fewer operand-bus toggles).
                 const int i = m / kTilesN, j = (i & 1) ? kTilesN - 1 - m % kTilesN : m % kTilesN;
                 acc[i][j] = Mfma<T>::run(frag_b[buffer][j], frag_a[buffer][i], acc[i][j]);  // transposed, see store_tile
-                if (m < 4) {
+                if constexpr (kHalf) {
+                    if (m < 4) read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
+                    else if (m < 6) read_lhs_fragment(last, next_kstep, buffer ^ 1, m - 4);
+                    // All rhs loads of a K-step before its lhs loads: the wait before the barrier counts on it.
+                    if (m >= 2 && m < 6) {
+                        if (kstep == 0) load_rhs.load(kNextSlot * kOperandBytes, 4 + m - 2);
+                        else if (last) load_rhs.load(kSlot * kOperandBytes, m - 2);
+                    }
+                    if (m >= 6) load_lhs.load(lhs_target, lhs_chunk + m - 6);
+                } else if (m < 4) {
                     read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
                 } else if (m < 8) {
                     read_lhs_fragment(last, next_kstep, buffer ^ 1, m - 4);
@@ -975,9 +997,16 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         // Two slices per trip (the rhs slots alternate); an odd count multiplies one slice of zeros. (Leaving the
         // loop before that slice costs far more than it saves: with a second exit the compiler no longer keeps the
         // accumulators in place and the kernel ran five times slower.)
-        for (int t = 0; t < num_slices; t += 2) {
-            iteration(t, slot0);
-            iteration(t + 1, slot1);
+        if (half_tile) {
+            for (int t = 0; t < num_slices; t += 2) {
+                iteration(t, slot0, std::true_type{});
+                iteration(t + 1, slot1, std::true_type{});
+            }
+        } else {
+            for (int t = 0; t < num_slices; t += 2) {
+                iteration(t, slot0, std::false_type{});
+                iteration(t + 1, slot1, std::false_type{});
+            }
         }
         wait_for_loads<0>();  // the zero-filling loads of slices past the end still write LDS
     }
@@ -1003,7 +1032,8 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             store_partial(acc, args.partials + static_cast<int64_t>(piece_slot) * kPartialFloats, wave, lane);
         else
             store_result(
-                args, work, [&](int i) -> const f32x16_t(&)[kTilesN] { return acc[i]; }, lds, wave, lane);
+                args, work, [&](int i) -> const f32x16_t(&)[kTilesN] { return acc[i]; }, lds, wave, lane, wave_row_base,
+                wave_row_blocks);
     }
 }
 
@@ -1048,7 +1078,7 @@ __global__ __launch_bounds__(64) void grouped_gemm_reduce_kernel(GemmArgs args) 
         }
         return block;
     };
-    store_result(args, work, summed_block, lds, wave, lane);
+    store_result(args, work, summed_block, lds, wave, lane, (wave / kWavesN) * kWaveRows, kTilesM);
 }
 
 // ---- host side -----------------------------------------------------------------------------------------
