@@ -12,7 +12,8 @@ bandwidth-bound kernels, the same step with fp32 gradient buffers, the other fou
 CPU baseline (the looped torch MoE on the host cores, on a bounded token sample).
 
 `python bench.py --ceilings` prints, instead, what the device sustains: back-to-back MFMAs on zero and on random
-operands, the vendor BLAS on dense products of the same sizes, and a plain streaming copy.
+operands, the vendor BLAS on dense products of the same sizes, a plain streaming copy, and the rate at which the CUs
+fill LDS from L2.
 """
 
 import argparse
@@ -292,6 +293,41 @@ def measure_ceilings(device: torch.device) -> dict:
     assert torch.equal(source, target)
     result["torch_copy_gbs"] = round(2 * size / timed(lambda: target.copy_(source), 20) / 1e6, 1)
     result["torch_add_gbs"] = round(2 * size / timed(lambda: torch.add(source, 1, out=target), 20) / 1e6, 1)
+    del source, target
+
+    # L2 -> LDS: every CU streams 64 KiB per iteration (one 256 x 256 x 64 bf16 slice) from a region that stays in its
+    # XCD's 4 MiB L2 (groups of 4 CUs share 256 KiB: 2 MiB per XCD; or all 32 CUs of an XCD share 1 MiB), and, for
+    # comparison, from regions that do not fit in L2 (4 MiB per CU).
+    iterations = 4000
+    cycles = torch.zeros(compute_units, dtype=torch.int64, device=device)
+    for name, region_bytes, shared_by, in_flight in (
+        ("l2_16_loads_in_flight", 256 << 10, 4, 1),
+        ("l2_32_loads_in_flight", 256 << 10, 4, 2),
+        ("l2_48_loads_in_flight", 256 << 10, 4, 3),
+        ("l2_shared_by_32_48_loads_in_flight", 1 << 20, 32, 3),
+        ("l2_48_loads_in_flight_64_cus", 256 << 10, 4, 3),
+        ("beyond_l2_48_loads_in_flight", 4 << 20, 1, 3),
+    ):
+        workgroups = 64 if name.endswith("64_cus") else compute_units
+        groups = 8 * -(-(workgroups // 8) // shared_by)
+        region = torch.empty(groups * region_bytes, dtype=torch.uint8, device=device).random_(0, 255)
+        ms = timed(
+            lambda: _lib.check(
+                library.fm_probe_l2(
+                    region.data_ptr(), region_bytes, shared_by, workgroups, iterations, in_flight, cycles.data_ptr(),
+                    stream.cuda_stream,
+                )
+            ),
+            3,
+        )
+        mean_cycles = cycles[:workgroups].double().mean().item()
+        result[f"lds_fill_from_{name}"] = {
+            "tbs": round(workgroups * iterations * 65536 / ms / 1e9, 2),
+            "bytes_per_cycle_per_cu": round(iterations * 65536 / mean_cycles, 1),
+            "shader_clock_mhz": round(mean_cycles / ms / 1e3),
+            "cycles_per_64_kib": round(mean_cycles / iterations),
+        }
+        del region
     result["peaks"] = {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "hbm_gbs": PEAK_HBM_GBS}
     return result
 

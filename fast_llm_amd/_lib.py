@@ -54,6 +54,7 @@ SIGNATURES: dict[str, tuple] = {
     "fm_probe_mfma": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_int, ctypes.c_float, _c_ptr]),
     "fm_probe_mfma_flops": (_c_i64, [_c_i64, _c_i64]),
     "fm_probe_copy": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
+    "fm_probe_l2": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),
 }
 
 FM_ERR_INVALID_ARGUMENT, FM_ERR_UNSUPPORTED, FM_ERR_LAUNCH = -1, -2, -3

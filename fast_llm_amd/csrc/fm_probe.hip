@@ -5,6 +5,10 @@
 //     bf16 values. The chip lowers its clock under power, and operand toggling costs power: the rate on random data
 //     is the ceiling a product on real activations can reach, the rate on zeros is the published peak.
 //   fm_probe_copy: a plain streaming copy (16-byte vectors, one read and one write per byte).
+//   fm_probe_l2: every workgroup streams a small region that stays in its XCD's L2 straight into LDS, 64 KiB per
+//     iteration (what a 256 x 256 x 64 bf16 GEMM slice needs), with the GEMM's load instruction. A workgroup tile of
+//     256 x 256 needs 1/128 byte per FLOP from L2, i.e. 32 bytes per cycle and CU at the matrix peak of 4096
+//     FLOP/cycle/CU: the rate measured here says how far below the matrix peak the L2 caps such a product.
 #include "fm_common.h"
 
 namespace fm {
@@ -74,7 +78,60 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const RawVec16 *__restr
         __builtin_nontemporal_store(__builtin_nontemporal_load(source + i), target + i);
 }
 
+// One workgroup per CU (the dynamic LDS leaves room for one). Workgroups b, b + 8, b + 16, ... run on the same XCD;
+// groups of `shared_by` of them stream the same region of `region_bytes`, 64 KiB per iteration, wrapping around.
+// kInFlight: iterations a wavefront may have on their way besides the one it is issuing (16 loads each).
+template <int kInFlight>
+__global__ __launch_bounds__(256, 1) void probe_l2_kernel(const char *base, int64_t region_bytes, int shared_by,
+                                                          int64_t iterations, int64_t *cycles) {
+    extern __shared__ __attribute__((aligned(1024))) char probe_lds_generic[];
+    __attribute__((address_space(3))) char *lds = (__attribute__((address_space(3))) char *)(probe_lds_generic);
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
+    const int groups_per_xcd = (gridDim.x / 8 + shared_by - 1) / shared_by;
+    const char *region = base + static_cast<int64_t>(xcd * groups_per_xcd + local / shared_by) * region_bytes;
+    // Members of a group start at different offsets so that they do not walk in lock step.
+    const uint32_t mask = static_cast<uint32_t>(region_bytes - 1);  // region_bytes is a power of two
+    uint32_t offset = static_cast<uint32_t>(local % shared_by) * 65536u & mask;
+    __syncthreads();
+    const int64_t start = clock64();
+    for (int64_t iteration = 0; iteration < iterations; ++iteration) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const char *pointer = region + (((offset + (wave * 16 + j) * 1024u) & mask) + lane * 16);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)pointer,
+                                             (__attribute__((address_space(3))) void *)(lds + (iteration & 1) * 65536 +
+                                                                                        (wave * 16 + j) * 1024),
+                                             16, 0, 0);
+        }
+        offset = (offset + 65536u) & mask;
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(16 * kInFlight) : "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) cycles[blockIdx.x] = clock64() - start;
+}
+
 }  // namespace fm
+
+extern "C" int fm_probe_l2(const void *source, int64_t region_bytes, int64_t shared_by, int64_t workgroups,
+                           int64_t iterations, int64_t in_flight, void *cycles, void *stream) {
+    using namespace fm;
+    FM_REQUIRE(source && cycles && aligned16(source), "fm_probe_l2: null or misaligned buffer");
+    FM_REQUIRE(region_bytes >= 65536 && region_bytes <= (int64_t(1) << 30) && (region_bytes & (region_bytes - 1)) == 0 &&
+                   shared_by > 0 && workgroups > 0 &&
+                   workgroups % 8 == 0 && workgroups < (1 << 20) && iterations >= 0 && in_flight >= 1 && in_flight <= 3,
+               "fm_probe_l2: regions are powers of two from 64 KiB to 1 GiB, workgroups a multiple of 8, 1 to 3 iterations in flight");
+    constexpr int kLdsBytes = 2 * 65536;
+    auto kernel = in_flight == 1 ? probe_l2_kernel<1> : in_flight == 2 ? probe_l2_kernel<2> : probe_l2_kernel<3>;
+    hipError_t error = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(error));
+    kernel<<<static_cast<int>(workgroups), 256, kLdsBytes, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const char *>(source), region_bytes, static_cast<int>(shared_by), iterations,
+        static_cast<int64_t *>(cycles));
+    return check_launch("fm_probe_l2");
+}
 
 extern "C" int fm_probe_mfma(void *sink, int64_t workgroups, int64_t iterations, int random_operands, float sigma,
                              void *stream) {

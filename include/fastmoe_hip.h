@@ -336,6 +336,15 @@ int64_t fm_probe_mfma_flops(int64_t workgroups, int64_t iterations);
  * 256 lanes (grid stride). `bytes` a multiple of 16, both pointers 16-byte aligned. */
 int fm_probe_copy(const void *source, void *target, int64_t bytes, int64_t workgroups, void *stream);
 
+/* `workgroups` workgroups (a multiple of 8, one per CU) of 4 wavefronts each stream 64 KiB per iteration from global
+ * memory straight into LDS with 16-byte loads, `iterations` times. Workgroups on one XCD form groups of `shared_by`
+ * that read the same region of `region_bytes` (a power of two, 64 KiB or more) over and over, so a small region stays in that
+ * XCD's L2. A wavefront keeps up to `in_flight` (1 to 3) iterations of 16 loads on their way while it issues the
+ * next. `source` holds (workgroups / 8 / shared_by rounded up) * 8 regions; `cycles` receives one int64 per
+ * workgroup: the shader clock cycles its loop took. */
+int fm_probe_l2(const void *source, int64_t region_bytes, int64_t shared_by, int64_t workgroups, int64_t iterations,
+                int64_t in_flight, void *cycles, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
