@@ -15,6 +15,10 @@
 namespace fm {
 
 constexpr int kCopyThreads = 256;
+// Gathered sparse rows are read once. While the sparse buffer fits the 256 MiB Infinity Cache, the rows the previous
+// kernel wrote are still there and ordinary loads find them (measured inside a training step at 142 MB: streaming loads
+// 2 % slower in the combine, 13 % in its backward); beyond that size streaming loads are faster (604 MB: 7 % and 3 %).
+constexpr int64_t kStreamGatherBytes = int64_t(256) << 20;
 
 struct CopyArgs {
     const void *sparse_rows;
@@ -24,6 +28,7 @@ struct CopyArgs {
     int experts_per_token;
     int index_dtype;
     int scores_dtype;
+    bool stream_gather;  // sparse rows are read with streaming loads (the sparse buffer is larger than the Infinity Cache)
 };
 
 __device__ __forceinline__ float load_score(const void *scores, int scores_dtype, int64_t i) {
@@ -80,7 +85,7 @@ __global__ __launch_bounds__(kCopyThreads) void copy_dense_to_sparse_kernel(cons
 // ---- combine -------------------------------------------------------------------------------------------
 // Slots are taken two at a time: all loads of a pair (and of all the lane's vectors) are issued before the first
 // addition; the additions keep the slot order j = 0 .. k - 1.
-template <typename T, bool kVector, int kChunks>
+template <typename T, bool kVector, int kChunks, bool kStreamGather = false>
 __global__ __launch_bounds__(kCopyThreads) void copy_sparse_to_dense_kernel(const T *__restrict__ input,
                                                                             T *__restrict__ output, CopyArgs args) {
     constexpr int N = kVector ? Vec16<T>::N : 1;
@@ -112,7 +117,9 @@ __global__ __launch_bounds__(kCopyThreads) void copy_sparse_to_dense_kernel(cons
                     for (int q = 0; q < kPasses; ++q) {
                         const int64_t c = c0 + q * stride;
                         if (c < columns) {
-                            if constexpr (kVector) value[u][q] = load16(input + row * columns + c);
+                            if constexpr (kVector)
+                                value[u][q] = kStreamGather ? load16_stream(input + row * columns + c)
+                                                            : load16(input + row * columns + c);
                             else value[u][q].v[0] = input[row * columns + c];
                         }
                     }
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(kCopyThreads) void copy_sparse_to_dense_kernel(cons
 // grad_scores[t, j] = <input[row(t, j), :], grad_output[t, :]>; when kFused also
 // grad_input[row(t, j), :] = grad_output[t, :] * scores[t, j].
 // kChunks vectors of grad_output per lane are kept in registers across the k slots.
-template <typename T, typename OutT, bool kVector, bool kFused, int kChunks>
+template <typename T, typename OutT, bool kVector, bool kFused, int kChunks, bool kStreamGather = false>
 __global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__restrict__ input,
                                                                   const T *__restrict__ grad_output,
                                                                   T *__restrict__ grad_input,
@@ -176,44 +183,8 @@ __global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__res
         }
     }
 
-    for (int j = 0; j < k; ++j) {
-        const int64_t row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
-        float score = 0.f;
-        if constexpr (kFused) score = load_score(args.scores, args.scores_dtype, token * k + j);
-        float partial = 0.f;
-        if (row >= 0 && row < args.num_rows_sparse) {
-            const T *in_row = input + row * columns;
-            T *out_row = kFused ? grad_input + row * columns : nullptr;
-            auto body = [&](const Vec16<T> &g, int64_t c) {
-                Vec16<T> value;
-                if constexpr (kVector) value = load16(in_row + c);
-                else value.v[0] = in_row[c];
-#pragma unroll
-                for (int i = 0; i < N; ++i) partial += to_float(value.v[i]) * to_float(g.v[i]);
-                if constexpr (kFused) {
-                    Vec16<T> scaled;
-#pragma unroll
-                    for (int i = 0; i < N; ++i) scaled.v[i] = from_float<T>(to_float(g.v[i]) * score);
-                    if constexpr (kVector) store16_stream(out_row + c, scaled);
-                    else out_row[c] = scaled.v[0];
-                }
-            };
-            if constexpr (kChunks > 0) {
-#pragma unroll
-                for (int q = 0; q < kChunks; ++q) {
-                    const int64_t c = (static_cast<int64_t>(q) * blockDim.x + threadIdx.x) * N;
-                    if (c < columns) body(grad[q], c);
-                }
-            } else {
-                for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns;
-                     c += static_cast<int64_t>(blockDim.x) * N) {
-                    Vec16<T> g;
-                    if constexpr (kVector) g = load16(grad_row + c);
-                    else g.v[0] = grad_row[c];
-                    body(g, c);
-                }
-            }
-        }
+    // The reduction of a slot's products over the workgroup, and the store of the result.
+    auto finish_slot = [&](int j, float partial) {
         partial = wave_sum(partial);
         if (lane == 0) lds_partial[wave] = partial;
         __syncthreads();
@@ -223,6 +194,89 @@ __global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__res
             grad_scores[token * k + j] = from_float<OutT>(total);
         }
         __syncthreads();
+    };
+    auto products = [&](const Vec16<T> &value, const Vec16<T> &g, float score, T *out, float &partial) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) partial += to_float(value.v[i]) * to_float(g.v[i]);
+        if constexpr (kFused) {
+            Vec16<T> scaled;
+#pragma unroll
+            for (int i = 0; i < N; ++i) scaled.v[i] = from_float<T>(to_float(g.v[i]) * score);
+            if constexpr (kVector) store16_stream(out, scaled);
+            else out[0] = scaled.v[0];
+        }
+    };
+
+    if constexpr (kChunks > 0) {
+        // The lane's vectors of slot j + 1 are requested before slot j is reduced (two barriers and an LDS round trip
+        // per slot): a slot's memory latency overlaps the previous slot's reduction.
+        struct Slot {
+            int64_t row;
+            float score;
+            Vec16<T> value[kChunks];
+        };
+        auto request = [&](int j, Slot &slot) {
+            slot.row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
+            slot.score = 0.f;
+            if constexpr (kFused) slot.score = load_score(args.scores, args.scores_dtype, token * k + j);
+            if (slot.row < 0 || slot.row >= args.num_rows_sparse) {
+                slot.row = -1;
+                return;
+            }
+            const T *in_row = input + slot.row * columns;
+#pragma unroll
+            for (int q = 0; q < kChunks; ++q) {
+                const int64_t c = (static_cast<int64_t>(q) * blockDim.x + threadIdx.x) * N;
+                if (c < columns) {
+                    if constexpr (kVector) slot.value[q] = kStreamGather ? load16_stream(in_row + c) : load16(in_row + c);
+                    else slot.value[q].v[0] = in_row[c];
+                }
+            }
+        };
+        auto process = [&](int j, const Slot &slot) {
+            float partial = 0.f;
+            if (slot.row >= 0) {
+                T *out_row = kFused ? grad_input + slot.row * columns : nullptr;
+#pragma unroll
+                for (int q = 0; q < kChunks; ++q) {
+                    const int64_t c = (static_cast<int64_t>(q) * blockDim.x + threadIdx.x) * N;
+                    if (c < columns) products(slot.value[q], grad[q], slot.score, out_row + c, partial);
+                }
+            }
+            finish_slot(j, partial);
+        };
+        Slot even, odd;
+        request(0, even);
+        for (int j = 0; j < k; j += 2) {
+            if (j + 1 < k) request(j + 1, odd);
+            process(j, even);
+            if (j + 2 < k) request(j + 2, even);
+            if (j + 1 < k) process(j + 1, odd);
+        }
+    } else {
+        for (int j = 0; j < k; ++j) {
+            const int64_t row = load_index(args.sparse_rows, args.index_dtype, token * k + j);
+            float score = 0.f;
+            if constexpr (kFused) score = load_score(args.scores, args.scores_dtype, token * k + j);
+            float partial = 0.f;
+            if (row >= 0 && row < args.num_rows_sparse) {
+                const T *in_row = input + row * columns;
+                T *out_row = kFused ? grad_input + row * columns : nullptr;
+                for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns;
+                     c += static_cast<int64_t>(blockDim.x) * N) {
+                    Vec16<T> g, value;
+                    if constexpr (kVector) {
+                        g = load16(grad_row + c);
+                        value = load16(in_row + c);
+                    } else {
+                        g.v[0] = grad_row[c];
+                        value.v[0] = in_row[c];
+                    }
+                    products(value, g, score, out_row + c, partial);
+                }
+            }
+            finish_slot(j, partial);
+        }
     }
 }
 
@@ -247,8 +301,26 @@ static int copy_threads(int64_t num_columns, int vector, int per_lane = 1) {
         else KERNEL<T, true, 0><<<rows, threads, 0, stream>>>(in, out, args);                                        \
     }
 FM_DEFINE_COPY_LAUNCHER(launch_dispatch, copy_dense_to_sparse_kernel)
-FM_DEFINE_COPY_LAUNCHER(launch_combine, copy_sparse_to_dense_kernel)
 #undef FM_DEFINE_COPY_LAUNCHER
+
+template <typename T>
+static void launch_combine(const T *in, T *out, int64_t rows, const CopyArgs &args, bool vectorised, int chunks,
+                           int threads, hipStream_t stream) {
+#define FM_LAUNCH_COMBINE(VEC, CHUNKS)                                                                       \
+    do {                                                                                                     \
+        if (args.stream_gather)                                                                              \
+            copy_sparse_to_dense_kernel<T, VEC, CHUNKS, true><<<rows, threads, 0, stream>>>(in, out, args);  \
+        else                                                                                                 \
+            copy_sparse_to_dense_kernel<T, VEC, CHUNKS, false><<<rows, threads, 0, stream>>>(in, out, args); \
+    } while (0)
+    if (!vectorised) copy_sparse_to_dense_kernel<T, false, 0><<<rows, threads, 0, stream>>>(in, out, args);
+    else if (chunks <= 1) FM_LAUNCH_COMBINE(true, 1);
+    else if (chunks <= 2) FM_LAUNCH_COMBINE(true, 2);
+    else if (chunks <= 4) FM_LAUNCH_COMBINE(true, 4);
+    else if (chunks <= 8) FM_LAUNCH_COMBINE(true, 8);
+    else FM_LAUNCH_COMBINE(true, 0);
+#undef FM_LAUNCH_COMBINE
+}
 
 // Vectors of `vector` elements a lane handles when `threads` lanes share a row.
 static int chunks_per_lane(int64_t num_columns, int vector, int threads) {
@@ -282,7 +354,8 @@ extern "C" int fm_copy_dense_to_sparse(const void *input, const void *scores, co
         return status;
     if (num_rows_dense == 0 || num_columns == 0 || num_experts_per_token == 0) return FM_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    CopyArgs args{sparse_rows, scores, num_columns, num_rows_sparse, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype};
+    CopyArgs args{sparse_rows, scores, num_columns, num_rows_sparse, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype,
+                  num_rows_sparse * num_columns * dtype_size(dtype) > kStreamGatherBytes};
     const int vector = 16 / dtype_size(dtype);
     const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(output);
     // Two vectors per lane (measured on MI355X, inside a training step: rows of 4 KiB go 7 % faster with 128 lanes x 2
@@ -307,7 +380,8 @@ extern "C" int fm_copy_sparse_to_dense(const void *input, const void *scores, co
         return status;
     if (num_rows_dense == 0 || num_columns == 0) return FM_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    CopyArgs args{sparse_rows, scores, num_columns, num_rows_sparse, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype};
+    CopyArgs args{sparse_rows, scores, num_columns, num_rows_sparse, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype,
+                  num_rows_sparse * num_columns * dtype_size(dtype) > kStreamGatherBytes};
     const int vector = 16 / dtype_size(dtype);
     const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(output);
     const int threads = copy_threads(num_columns, vectorised ? vector : 1, 2);
@@ -331,8 +405,13 @@ static void launch_grad_score(const void *input, const void *grad_output, void *
     const int vector = vectorised ? Vec16<T>::N : 1;
     const int64_t chunks = (args.num_columns + static_cast<int64_t>(vector) * threads - 1) /
                            (static_cast<int64_t>(vector) * threads);
-#define FM_LAUNCH_GS(VEC, CHUNKS) \
-    grad_score_kernel<T, OutT, VEC, kFused, CHUNKS><<<rows, threads, 0, stream>>>(in, go, gi, gs, args)
+#define FM_LAUNCH_GS(VEC, CHUNKS)                                                                                   \
+    do {                                                                                                            \
+        if (args.stream_gather && CHUNKS > 0)                                                                       \
+            grad_score_kernel<T, OutT, VEC, kFused, CHUNKS, true><<<rows, threads, 0, stream>>>(in, go, gi, gs, args); \
+        else                                                                                                        \
+            grad_score_kernel<T, OutT, VEC, kFused, CHUNKS, false><<<rows, threads, 0, stream>>>(in, go, gi, gs, args); \
+    } while (0)
     if (vectorised) {
         if (chunks <= 1) FM_LAUNCH_GS(true, 1);
         else if (chunks <= 2) FM_LAUNCH_GS(true, 2);
@@ -357,7 +436,8 @@ static int grad_score_entry(const char *name, const void *input, const void *gra
     FM_REQUIRE(grad_scores, "%s: null grad_scores", name);
     if (kFused) FM_REQUIRE(scores && (grad_input || num_columns == 0), "%s: null scores or grad_input", name);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    CopyArgs args{sparse_rows, scores, num_columns, num_rows_sparse, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype};
+    CopyArgs args{sparse_rows, scores, num_columns, num_rows_sparse, static_cast<int>(num_experts_per_token), index_dtype, scores_dtype,
+                  num_rows_sparse * num_columns * dtype_size(dtype) > kStreamGatherBytes};
     const int vector = 16 / dtype_size(dtype);
     const bool vectorised = num_columns % vector == 0 && aligned16(input) && aligned16(grad_output) &&
                             (!kFused || aligned16(grad_input));
