@@ -101,12 +101,21 @@ __global__ __launch_bounds__(kMapBlock) void sparse_map_layout_kernel(int32_t *_
     // Exclusive prefix over workgroups of this expert's counts, in place.
     int64_t count = 0;
     if (e < num_experts) {
+        // 16 counts are requested before the first is used: one memory latency per 16 workgroups, not per workgroup
+        // (a load after a store to the same array is not moved ahead of it by the compiler).
+        constexpr int kBatch = 16;
         int32_t running = 0;
-        for (int b = 0; b < num_blocks; ++b) {
-            int32_t *slot = block_counts + static_cast<int64_t>(b) * num_experts + e;
-            const int32_t here = *slot;
-            *slot = running;
-            running += here;
+        for (int b0 = 0; b0 < num_blocks; b0 += kBatch) {
+            int32_t *slot = block_counts + static_cast<int64_t>(b0) * num_experts + e;
+            int32_t here[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i)
+                here[i] = b0 + i < num_blocks ? slot[static_cast<int64_t>(i) * num_experts] : 0;
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                if (b0 + i < num_blocks) slot[static_cast<int64_t>(i) * num_experts] = running;
+                running += here[i];
+            }
         }
         count = running;
     }
@@ -124,17 +133,27 @@ __global__ __launch_bounds__(kMapBlock) void sparse_map_layout_from_router_kerne
     const int e = threadIdx.x;
     int64_t count = 0;
     if (e < num_experts) {
+        constexpr int kBatch = 16;  // counts requested together, as in sparse_map_layout_kernel
         int32_t running = 0;
-        for (int b = 0; b < num_blocks; ++b) {
-            int32_t here;
-            if (e < routed_experts) {
-                here = static_cast<int32_t>(router_partials[static_cast<int64_t>(b) * router_stats + routed_experts + e]);
-            } else {
-                const int64_t begin = b * tokens_per_block;
-                here = static_cast<int32_t>(max(int64_t(0), min(begin + tokens_per_block, num_tokens) - begin));
+        for (int b0 = 0; b0 < num_blocks; b0 += kBatch) {
+            int32_t here[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                const int b = b0 + i;
+                if (b >= num_blocks) {
+                    here[i] = 0;
+                } else if (e < routed_experts) {
+                    here[i] = static_cast<int32_t>(router_partials[static_cast<int64_t>(b) * router_stats + routed_experts + e]);
+                } else {
+                    const int64_t begin = b * tokens_per_block;
+                    here[i] = static_cast<int32_t>(max(int64_t(0), min(begin + tokens_per_block, num_tokens) - begin));
+                }
             }
-            block_prefix[static_cast<int64_t>(b) * num_experts + e] = running;
-            running += here;
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                if (b0 + i < num_blocks) block_prefix[static_cast<int64_t>(b0 + i) * num_experts + e] = running;
+                running += here[i];
+            }
         }
         count = running;
     }
