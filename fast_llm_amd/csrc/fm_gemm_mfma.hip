@@ -467,7 +467,9 @@ __device__ __forceinline__ int count_row_tiles(const GemmArgs &args) {
     return __builtin_amdgcn_readfirstlane(tiles);
 }
 
-__device__ __forceinline__ SplitPlan plan_split(const GemmArgs &args) {
+// `with_pieces` false: only tiles_m, whole and tail are wanted (what a workgroup of the whole tiles needs to know; the
+// search for the best cut is a dozen integer divisions).
+__device__ __forceinline__ SplitPlan plan_split(const GemmArgs &args, bool with_pieces = true) {
     SplitPlan plan;
     plan.tiles_m = count_row_tiles(args);
     const int total = plan.tiles_m * args.tiles_n;
@@ -477,7 +479,7 @@ __device__ __forceinline__ SplitPlan plan_split(const GemmArgs &args) {
     const int num_slices = static_cast<int>(args.inner / kBK);
     plan.piece_slices = num_slices;
     int best = num_slices;
-    if (plan.tail > 0) {
+    if (plan.tail > 0 && with_pieces) {
 #pragma unroll
         for (int split = 2; split <= 8; split *= 2) {
             if (plan.tail * split > kMaxPartials || num_slices / split < kMinPieceSlices) continue;
@@ -503,8 +505,9 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int
     piece_slices = 0;
     piece_slot = -1;
     if (args.partials == nullptr) return true;
-    const SplitPlan plan = plan_split(args);
+    SplitPlan plan = plan_split(args, false);
     if (logical >= plan.whole) {
+        plan = plan_split(args);
         const int index = logical - plan.whole;
         if (index >= plan.tail * plan.pieces) return false;
         if (plan.pieces > 1) {
@@ -849,12 +852,14 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     }
 
     f32x16_t acc[kTilesM][kTilesN];
+    auto clear_accumulators = [&]() {
 #pragma unroll
-    for (int i = 0; i < kTilesM; ++i)
+        for (int i = 0; i < kTilesM; ++i)
 #pragma unroll
-        for (int j = 0; j < kTilesN; ++j)
+            for (int j = 0; j < kTilesN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    };
 
     // ---- the software pipeline --------------------------------------------------------------------------
     // A slot that is being filled cannot be read, and LDS (160 KiB) has room for five operand slices of 32 KiB: three
@@ -984,6 +989,7 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         load_lhs.advance();
 #pragma unroll
         for (int j = 0; j < 2; ++j) load_lhs.load(lhs_after, j);
+        clear_accumulators();  // 256 register writes, while the first loads are on their way
         wait_for_loads<14>();  // 30 loads so far, the first 16 of them slice 0
         __syncthreads();
         mask_slice(0, lhs_now, 0);
@@ -1009,6 +1015,8 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             }
         }
         wait_for_loads<0>();  // the zero-filling loads of slices past the end still write LDS
+    } else {
+        clear_accumulators();
     }
 
     if (piece_slot < 0 && args.accumulate != 0 && num_slices == 0) return;  // nothing to add
