@@ -43,6 +43,7 @@ SIGNATURES: dict[str, tuple] = {
     "fm_mlp_activation_forward": (_c_int, [_c_ptr] * 2 + [_c_i64] * 2 + [_c_int] * 3 + [_c_ptr, _c_int, _c_ptr]),
     "fm_mlp_activation_backward": (_c_int, [_c_ptr] * 4 + [_c_i64] * 2 + [_c_int] * 3 + [_c_ptr, _c_int, _c_ptr]),
     "fm_grouped_gemm_workspace_size": (_c_size, [_c_i64] * 4 + [_c_int]),
+    "fm_input_row_sparse_matmul_workspace_size": (_c_size, [_c_i64] * 4 + [_c_int]),
     "fm_output_sparse_matmul": (_c_int, [_c_ptr] * 4 + [_c_i64] * 10 + [_c_int] * 4 + [_c_ptr, _c_size, _c_ptr]),
     "fm_input_inner_sparse_matmul": (_c_int, [_c_ptr] * 4 + [_c_i64] * 10 + [_c_int] * 4 + [_c_ptr, _c_size, _c_ptr]),
     "fm_input_row_sparse_matmul": (_c_int, [_c_ptr] * 5 + [_c_i64] * 10 + [_c_int] * 4 + [_c_ptr, _c_size, _c_ptr]),

@@ -243,17 +243,28 @@ extern "C" int fm_input_row_sparse_matmul(const void *lhs, const void *rhs, void
     return run_gemm("fm_input_row_sparse_matmul", args, dtype, workspace, workspace_size, stream);
 }
 
-extern "C" size_t fm_grouped_gemm_workspace_size(int64_t row_dim, int64_t col_dim, int64_t inner_dim,
-                                                 int64_t num_experts, int dtype) {
-    if (dtype != FM_DTYPE_BF16 && dtype != FM_DTYPE_F16) return 0;  // fp32 operands never take the splitting kernel
+static size_t workspace_size_of(int mode, int64_t row_dim, int64_t col_dim, int64_t inner_dim, int64_t num_experts,
+                                int dtype) {
+    if (dtype != FM_DTYPE_BF16 && dtype != FM_DTYPE_F16) return 0;  // fp32 operands never take the matrix-core kernel
     if (row_dim <= 0 || col_dim <= 0 || inner_dim <= 0 || num_experts < 0 || num_experts >= (1 << 20)) return 0;
     GemmArgs args{};
-    args.rows = row_dim;
+    args.num_experts = static_cast<int>(num_experts > 1 ? num_experts : 1);
+    args.rows = mode == kInputRowSparse ? row_dim * args.num_experts : row_dim;
     args.cols = col_dim;
     args.inner = inner_dim;
-    args.num_experts = static_cast<int>(num_experts > 1 ? num_experts : 1);
-    args.mode = kOutputSparse;  // the input-inner-sparse product tiles the same way
+    args.sparse_size = mode == kInputRowSparse ? row_dim : 0;
+    args.mode = mode;
     return mfma_gemm_workspace_size(args);
+}
+
+extern "C" size_t fm_grouped_gemm_workspace_size(int64_t row_dim, int64_t col_dim, int64_t inner_dim,
+                                                 int64_t num_experts, int dtype) {
+    return workspace_size_of(kOutputSparse, row_dim, col_dim, inner_dim, num_experts, dtype);  // input-inner-sparse: same
+}
+
+extern "C" size_t fm_input_row_sparse_matmul_workspace_size(int64_t row_sparse_dim, int64_t col_dim, int64_t inner_dim,
+                                                            int64_t num_experts, int dtype) {
+    return workspace_size_of(kInputRowSparse, row_sparse_dim, col_dim, inner_dim, num_experts, dtype);
 }
 
 // ---- grouped products with the gated activation fused into the epilogue ------------------------------------

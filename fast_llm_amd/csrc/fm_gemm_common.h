@@ -40,6 +40,8 @@ struct GemmArgs {
     void *fused_out;
     int64_t fused_stride;  // row stride of fused_out, elements
     int64_t half;          // columns of the activation output per expert
+    int num_ids;           // workgroup ids that may have a tile (set by the MFMA kernel's launcher)
+    void *tile_table;      // one record per id, written by the plan kernel into the caller's workspace, or null
 };
 
 template <typename OutT>

@@ -27,8 +27,11 @@
 //     full 256-byte row segments.
 //   * Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are renumbered so that the tiles an XCD
 //     runs at the same time are about 8 row tiles x 4 column tiles of one expert, which re-read operands from its L2.
-//   * When a launch has few rounds of long tiles and the caller brings a workspace, the reductions of the last
-//     round's tiles are split over the idle CUs and a second kernel adds the pieces in a fixed order.
+//   * The grid is one workgroup per CU; a workgroup walks its share of the tiles and issues the first loads of a
+//     tile before it writes the previous one out. With a workspace from the caller, where a tile lies is looked up
+//     in a table that a small kernel fills first (one scalar load instead of a scan of the expert map per tile),
+//     and, when a launch has few rounds of long tiles, the reductions of the last round's tiles are split over the
+//     idle CUs and a second kernel adds the pieces in a fixed order.
 // Results are deterministic: one workgroup per output tile (or a fixed split), fixed summation order, no atomics.
 #include <type_traits>
 
@@ -95,8 +98,11 @@ constexpr int kLoadsPerOperand = kOperandBytes / 16 / kMfmaThreads;  // 16-byte 
 constexpr int kBufferResourceFlags = 0x00020000;  // raw buffer, 32-bit data format, no swizzle
 constexpr int kEpiloguePadBytes = 16;  // after each staged row of the epilogue; keeps 16-byte alignment and spreads
                                        // the rows over the banks
+constexpr int kStagingBase = kOperandBytes;  // the epilogue stages rows in LDS from here up to the last lhs slot
 static_assert(kBK == 64 && kLoadsPerOperand == 8, "pipeline shape");
-static_assert(kLdsBytes <= 160 * 1024 && kWaves * 32 * (kWaveCols * 4 + kEpiloguePadBytes) <= kLdsBytes, "LDS budget");
+static_assert(kLdsBytes <= 160 * 1024 && kStagingBase + kWaves * 32 * (kWaveCols * 4 + kEpiloguePadBytes) <=
+                                             kLdsBytes - kOperandBytes,
+              "LDS budget: staging between rhs slot 0 and the last lhs slot");
 
 // ---- LDS layouts ---------------------------------------------------------------------------------------
 // K-contiguous operand, [256 rows][kBK k]: 16-byte chunk c (8 k values) of row r sits at
@@ -114,6 +120,13 @@ __device__ __forceinline__ int lds_offset_row_major(int k, int row) {
     return k * (kTile * 2) + ((((row >> 4) ^ ((k & 3) << 1)) << 5) | ((row & 15) << 1));
 }
 
+// The same value, but the compiler cannot tell: what is computed from it is computed where it is written, not hoisted
+// out of an enclosing loop into registers that stay occupied across the loop.
+__device__ __forceinline__ int opaque(int value) {
+    asm volatile("" : "+v"(value));
+    return value;
+}
+
 // Tell the compiler that a pointer computed from tile coordinates is the same in every lane (it then lives in
 // scalar registers and the loads use the scalar-base addressing form).
 __device__ __forceinline__ const char *uniform_pointer(const char *pointer) {
@@ -121,6 +134,12 @@ __device__ __forceinline__ const char *uniform_pointer(const char *pointer) {
     const uint32_t low = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
     const uint32_t high = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
     return reinterpret_cast<const char *>((static_cast<uint64_t>(high) << 32) | low);
+}
+
+__device__ __forceinline__ int64_t uniform_int64(int64_t value) {
+    const uint32_t low = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(value));
+    const uint32_t high = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(static_cast<uint64_t>(value) >> 32));
+    return static_cast<int64_t>((static_cast<uint64_t>(high) << 32) | low);
 }
 
 // Loader of one operand slice: global memory -> LDS, without passing through registers (`buffer_load ... lds`: lane
@@ -247,7 +266,7 @@ __device__ __forceinline__ u32x4_t load_fragment(FM_LDS(char) * lds, const int (
 // outside [k_lo, k_hi). Runs between two barriers, for the first/last slice of a ragged reduction range only.
 template <bool kContiguousK>
 __device__ __forceinline__ void mask_tile(FM_LDS(char) * operand_lds, int k0, int k_lo, int k_hi) {
-    for (int slot = threadIdx.x; slot < kOperandBytes / 16; slot += kMfmaThreads) {
+    for (int slot = opaque(static_cast<int>(threadIdx.x)); slot < kOperandBytes / 16; slot += kMfmaThreads) {
         FM_LDS(u32x4_t) *pointer = reinterpret_cast<FM_LDS(u32x4_t) *>(operand_lds + slot * 16);
         if constexpr (kContiguousK) {
             const int row = slot / kChunksPerRow;
@@ -324,7 +343,7 @@ __device__ __forceinline__ bool locate_tile(const GemmArgs &args, int logical, R
         tile.rows_valid = static_cast<int>(min(static_cast<int64_t>(kTile), args.rows - tile.row0));
         return true;
     }
-    const int lane = threadIdx.x & 63;
+    const int lane = opaque(static_cast<int>(threadIdx.x & 63));
     int tiles_before = 0;  // row tiles of the experts before this block of 64
     for (int base = 0; base < args.num_experts; base += 64) {
         const int e = base + lane;
@@ -450,7 +469,7 @@ struct SplitPlan {
 // sum over experts of ceil(rows_e / 256). Wave-uniform.
 __device__ __forceinline__ int count_row_tiles(const GemmArgs &args) {
     if (args.expert_ends == nullptr) return static_cast<int>((args.rows + kTile - 1) / kTile);
-    const int lane = threadIdx.x & 63;
+    const int lane = opaque(static_cast<int>(threadIdx.x & 63));
     int tiles = 0;
     for (int base = 0; base < args.num_experts; base += 64) {
         const int e = base + lane;
@@ -518,6 +537,58 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs &args, int pid, int
         }
     }
     return true;
+}
+
+// ---- the tile table -----------------------------------------------------------------------------------------
+// What a workgroup needs to know about the tile of an id: found by `compute_tile_record` from the expert map (a scan
+// of `expert_ends` with lane shuffles, a few integer divisions, a few thousand cycles), either by the workgroup itself
+// or, when the caller brings a workspace, once per launch by `grouped_gemm_plan_kernel`, which leaves one record per id
+// in a table that the workgroups then read with one scalar load per tile.
+struct alignas(64) TileRecord {
+    int64_t lhs_offset, rhs_offset, out_offset, fused_offset;  // elements
+    int rows_valid, cols_valid;
+    int k_lo, k_hi;    // reduction range (a piece of it for a split tile; ragged for the row-sparse product)
+    int piece_slot;    // >= 0: a piece of a split reduction, stored to that workspace slot
+    int found;         // 0: the id has no tile (and no later id has one)
+    int unused[2];
+};
+static_assert(sizeof(TileRecord) == 64, "one s_load_dwordx16 per record");
+
+// Wave-uniform result; every lane of the wavefront must call it.
+__device__ __forceinline__ bool compute_tile_record(const GemmArgs &args, int id, TileRecord &record) {
+    int logical, piece, piece_slices, piece_slot;
+    TileWork work;
+    const bool found = tile_of_block(args, id, logical, piece, piece_slices, piece_slot) && resolve_tile(args, logical, work);
+    record.found = __builtin_amdgcn_readfirstlane(found);
+    if (!record.found) return false;
+    record.piece_slot = __builtin_amdgcn_readfirstlane(piece_slot);
+    if (record.piece_slot >= 0) {  // a piece of a tile whose reduction is split (never the row-sparse product)
+        work.k_lo = static_cast<int64_t>(piece) * piece_slices * kBK;
+        work.k_hi = min(work.k_hi, work.k_lo + static_cast<int64_t>(piece_slices) * kBK);
+    }
+    record.lhs_offset = uniform_int64(work.lhs_offset);
+    record.rhs_offset = uniform_int64(work.rhs_offset);
+    record.out_offset = uniform_int64(work.out_offset);
+    record.fused_offset = uniform_int64(work.fused_offset);
+    record.rows_valid = __builtin_amdgcn_readfirstlane(work.rows_valid);
+    record.cols_valid = __builtin_amdgcn_readfirstlane(work.cols_valid);
+    record.k_lo = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_lo));
+    record.k_hi = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_hi));
+    return true;
+}
+
+// One wavefront per id.
+__global__ __launch_bounds__(256) void grouped_gemm_plan_kernel(GemmArgs args, TileRecord *table) {
+    const int id = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (id >= args.num_ids) return;
+    TileRecord record;
+    record.unused[0] = record.unused[1] = 0;
+    if (!compute_tile_record(args, id, record)) {
+        record.lhs_offset = record.rhs_offset = record.out_offset = record.fused_offset = 0;
+        record.rows_valid = record.cols_valid = record.k_lo = record.k_hi = 0;
+        record.piece_slot = -1;
+    }
+    if ((threadIdx.x & 63) == 0) table[id] = record;
 }
 
 // ---- the kernel ----------------------------------------------------------------------------------------
@@ -760,8 +831,8 @@ __device__ __forceinline__ void store_tile_gated_forward(const f32x16_t (&acc)[k
     }
 }
 
-template <typename Source>
-__device__ __forceinline__ void store_result(const GemmArgs &args, const TileWork &work, Source &&source,
+template <typename Work, typename Source>
+__device__ __forceinline__ void store_result(const GemmArgs &args, const Work &work, Source &&source,
                                              FM_LDS(char) * lds, int wave, int lane, int row_base, int blocks) {
     const bool accumulate = args.accumulate != 0;
     auto store = [&](auto *out) {
@@ -804,52 +875,66 @@ __device__ __forceinline__ void store_partial(const f32x16_t (&acc)[kTilesM][kTi
 // kMasked: the row-sparse product, whose reduction range [k_lo, k_hi) is ragged.
 // kFusion: a GemmFusion, the epilogue to run instead of the plain store.
 template <typename T, bool kLhsContiguousK, bool kRhsContiguousK, bool kMasked, int kFusion = kFusionNone>
-__global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_kernel(GemmArgs args) {
+__global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_kernel(GemmArgs launch_args) {
     static_assert(kFusion == kFusionNone || (kRhsContiguousK && !kMasked), "fused epilogues: output-sparse, K-major rhs");
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);  // C-style: address-space cast
-
-    int logical, piece, piece_slices, piece_slot;
-    TileWork work;
-    if (!tile_of_block(args, blockIdx.x, logical, piece, piece_slices, piece_slot) || !resolve_tile(args, logical, work))
-        return;
-    piece_slot = __builtin_amdgcn_readfirstlane(piece_slot);
-    if (piece_slot >= 0) {  // a piece of a tile whose reduction is split (never the row-sparse product)
-        work.k_lo = static_cast<int64_t>(piece) * piece_slices * kBK;
-        work.k_hi = min(work.k_hi, work.k_lo + static_cast<int64_t>(piece_slices) * kBK);
-    }
+    // The arguments are read from the kernel-argument segment where they are needed, through a pointer the compiler
+    // cannot see through, and read again after the main loop (`forget_arguments`): otherwise it keeps all of them in
+    // scalar registers across the main loop, which then no longer fit.
+    typedef const __attribute__((address_space(4))) GemmArgs *ArgumentPointer;
+    ArgumentPointer argument_pointer = (ArgumentPointer)__builtin_amdgcn_kernarg_segment_ptr();
+    auto forget_arguments = [&]() { asm volatile("" : "+s"(argument_pointer)); };
+    forget_arguments();
+#define args (*(const GemmArgs *)argument_pointer)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wave_m = wave / kWavesN, wave_n = wave % kWavesN;
-    // Tile coordinates are the same in every lane; say so, so that they live in scalar registers.
-    work.k_lo = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_lo));
-    work.k_hi = __builtin_amdgcn_readfirstlane(static_cast<int>(work.k_hi));
-    work.rows_valid = __builtin_amdgcn_readfirstlane(work.rows_valid);
-    work.cols_valid = __builtin_amdgcn_readfirstlane(work.cols_valid);
-    const int64_t k_first = work.k_lo / kBK * kBK;
-    const int64_t k_last = work.k_hi > work.k_lo ? (work.k_hi + kBK - 1) / kBK * kBK : k_first;
-    const int num_slices = __builtin_amdgcn_readfirstlane(static_cast<int>((k_last - k_first) / kBK));
-    // A tile with at most 128 valid rows (the last row tile of an expert whose padded row count is an odd multiple of
-    // 128) is a half tile: the wavefronts share its 128 rows, 64 each, and issue half the MFMAs. The transfers stay as
-    // they are (the rows past the valid ones bring zeros or repeats that nobody reads).
-    const bool half_tile = kFusion == kFusionNone && piece_slot < 0 && work.rows_valid <= kTile / 2;  // wave-uniform
-    const int wave_row_base = wave_m * (half_tile ? kWaveRows / 2 : kWaveRows);
-    const int wave_row_blocks = half_tile ? kTilesM / 2 : kTilesM;
+
+    // ---- the tiles of this workgroup ---------------------------------------------------------------------
+    // Workgroup b computes the tiles of the ids b, b + gridDim.x, b + 2 gridDim.x, ... below args.num_ids. With one
+    // workgroup per id that is one tile; with one workgroup per CU (a persistent grid) it is the sequence the hardware
+    // would hand that CU if all tiles took the same time, and the first loads of a tile are issued before the
+    // previous tile is written out. Ids map to tiles in increasing order, so the first id without a tile ends the walk.
+    // Everything about a tile is the same in every lane and is said to be, so that it lives in scalar registers.
+    struct Tile {
+        TileRecord work;
+        int piece_slot;   // >= 0: a piece of a split reduction, stored to that workspace slot
+        int k_first;      // first reduction index of slice 0 (a multiple of kBK)
+        int num_slices;
+        bool half;        // at most 128 valid rows: the wavefronts share them, 64 each, and issue half the MFMAs
+    };
+    auto find_tile = [&](int id, Tile &tile) -> bool {
+        if (args.tile_table != nullptr) {
+            // One scalar load (the table was written by an earlier kernel, so the scalar cache cannot hold stale lines).
+            typedef __attribute__((__vector_size__(16 * sizeof(uint32_t)))) uint32_t u32x16_t;
+            const TileRecord *address = static_cast<const TileRecord *>(args.tile_table) + id;
+            u32x16_t raw;
+            asm volatile("s_load_dwordx16 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(raw) : "s"(address) : "memory");
+            tile.work = __builtin_bit_cast(TileRecord, raw);
+            if (!tile.work.found) return false;
+        } else if (!compute_tile_record(args, id, tile.work)) {
+            return false;
+        }
+        const TileRecord &work = tile.work;
+        tile.piece_slot = work.piece_slot;
+        tile.k_first = work.k_lo / kBK * kBK;
+        const int k_last = work.k_hi > work.k_lo ? (work.k_hi + kBK - 1) / kBK * kBK : tile.k_first;
+        tile.num_slices = (k_last - tile.k_first) / kBK;
+        // A tile with at most 128 valid rows (the last row tile of an expert whose padded row count is an odd multiple
+        // of 128) is a half tile. The transfers stay as they are (the rows past the valid ones bring zeros or repeats
+        // that nobody reads).
+        tile.half = kFusion == kFusionNone && tile.piece_slot < 0 && work.rows_valid <= kTile / 2;
+        return true;
+    };
+
+    int id = blockIdx.x;
+    Tile tile;
+    if (id >= args.num_ids || !find_tile(id, tile)) return;
 
     TileLoader<kLhsContiguousK> load_lhs;
     TileLoader<kRhsContiguousK> load_rhs;
-    {
-        const char *lhs = static_cast<const char *>(args.lhs) +
-                          (work.lhs_offset + k_first * args.lhs_stride_inner) * static_cast<int64_t>(sizeof(T));
-        const char *rhs = static_cast<const char *>(args.rhs) +
-                          (work.rhs_offset + k_first * args.rhs_stride_inner) * static_cast<int64_t>(sizeof(T));
-        load_lhs.setup(uniform_pointer(lhs), (kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner) * sizeof(T),
-                       work.rows_valid, num_slices, wave, lane);
-        load_rhs.setup(uniform_pointer(rhs), (kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner) * sizeof(T),
-                       work.cols_valid, num_slices, wave, lane,
-                       kFusion == kFusionGatedForward ? static_cast<int>(args.half) : 0);
-    }
 
     f32x16_t acc[kTilesM][kTilesN];
     auto clear_accumulators = [&]() {
@@ -880,15 +965,10 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     constexpr int kLhsBase = kStages * kOperandBytes;  // LDS byte address of lhs slot 0; the rhs slots start at 0
     // LDS byte addresses of the lhs slots of slices t, t + 1, t + 2 (wave-uniform, rotated after every slice) and the
     // fragment addresses of this lane in the first two.
-    int lhs_now = kLhsBase, lhs_next = kLhsBase + kOperandBytes, lhs_after = kLhsBase + 2 * kOperandBytes;
+    // A tile starts with slice 0 in the LAST lhs slot and in rhs slot 0, so that the LDS in between, kStagingBase up to
+    // that lhs slot, is free for the previous tile's epilogue while those first loads are on their way.
+    int lhs_now, lhs_next, lhs_after;
     int lhs_frag0[4], lhs_frag[4], lhs_frag_next[4], rhs_frag[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        lhs_frag0[q] = fragment_base<kLhsContiguousK>(wave_row_base, q, lane);
-        lhs_frag[q] = lhs_frag0[q] + lhs_now;
-        lhs_frag_next[q] = lhs_frag0[q] + lhs_next;
-        rhs_frag[q] = fragment_base<kRhsContiguousK>(wave_n * kWaveCols, q, lane);
-    }
     auto read_rhs_fragment = [&](int slot, int kstep, int buffer, int j) {
         frag_b[buffer][j] = load_fragment<kRhsContiguousK>(lds, rhs_frag, slot, j, kstep);
     };
@@ -898,10 +978,11 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     };
     auto mask_slice = [&](int slice, int lhs_address, int rhs_slot) {
         if constexpr (kMasked) {
-            const int k0 = static_cast<int>(k_first) + slice * kBK;
-            if (slice < num_slices && (k0 < work.k_lo || k0 + kBK > work.k_hi)) {  // wave-uniform
-                mask_tile<kLhsContiguousK>(lds + lhs_address, k0, work.k_lo, work.k_hi);
-                mask_tile<kRhsContiguousK>(lds + rhs_slot * kOperandBytes, k0, work.k_lo, work.k_hi);
+            const int k_lo = tile.work.k_lo, k_hi = tile.work.k_hi;
+            const int k0 = tile.k_first + slice * kBK;
+            if (slice < tile.num_slices && (k0 < k_lo || k0 + kBK > k_hi)) {  // wave-uniform
+                mask_tile<kLhsContiguousK>(lds + lhs_address, k0, k_lo, k_hi);
+                mask_tile<kRhsContiguousK>(lds + rhs_slot * kOperandBytes, k0, k_lo, k_hi);
                 __syncthreads();
             }
         }
@@ -974,12 +1055,52 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             lhs_frag_next[q] = lhs_frag0[q] + lhs_next;
         }
     };
-    if (num_slices > 0) {
-        // Prologue: slice 0, lhs slice 1 and the first pieces of the slices after them on their way; slice 0 landed.
+    // The loads that start a tile come in two parts: slice 0 of both operands (16 loads per wavefront), which are issued
+    // while the previous tile is still being written out, and the 14 loads that follow (lhs slice 1, rhs chunks 0..3
+    // of slice 1, lhs chunks 0, 1 of slice 2). Nothing that `first_loads` computes per lane outlives it: the loaders
+    // and fragment addresses of the tile are set up (again) by `setup_tile`, after the previous tile's epilogue, so
+    // that they do not occupy registers during it.
+    auto setup_loaders = [&](const Tile &next, TileLoader<kLhsContiguousK> &lhs_loader,
+                             TileLoader<kRhsContiguousK> &rhs_loader, int lane) {
+        const TileRecord &work = next.work;
+        const char *lhs = static_cast<const char *>(args.lhs) +
+                          (work.lhs_offset + next.k_first * args.lhs_stride_inner) * static_cast<int64_t>(sizeof(T));
+        const char *rhs = static_cast<const char *>(args.rhs) +
+                          (work.rhs_offset + next.k_first * args.rhs_stride_inner) * static_cast<int64_t>(sizeof(T));
+        lhs_loader.setup(uniform_pointer(lhs),
+                         (kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner) * sizeof(T), work.rows_valid,
+                         next.num_slices, wave, lane);
+        rhs_loader.setup(uniform_pointer(rhs),
+                         (kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner) * sizeof(T), work.cols_valid,
+                         next.num_slices, wave, lane, kFusion == kFusionGatedForward ? static_cast<int>(args.half) : 0);
+    };
+    constexpr int kFirstLhsSlot = kLhsBase + (kLhsStages - 1) * kOperandBytes;
+    auto first_loads = [&](const Tile &next) {
+        if (next.num_slices <= 0) return;
+        TileLoader<kLhsContiguousK> lhs_loader;
+        TileLoader<kRhsContiguousK> rhs_loader;
+        setup_loaders(next, lhs_loader, rhs_loader, opaque(lane));
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load(lhs_now, j);
+        for (int j = 0; j < kLoadsPerOperand; ++j) lhs_loader.load(kFirstLhsSlot, j);
 #pragma unroll
-        for (int j = 0; j < kLoadsPerOperand; ++j) load_rhs.load(0, j);
+        for (int j = 0; j < kLoadsPerOperand; ++j) rhs_loader.load(0, j);
+    };
+    auto setup_tile = [&](const Tile &next) {
+        const int lane = opaque(static_cast<int>(threadIdx.x & 63));
+        setup_loaders(next, load_lhs, load_rhs, lane);
+        lhs_now = kFirstLhsSlot;
+        lhs_next = kLhsBase;
+        lhs_after = kLhsBase + kOperandBytes;
+        const int wave_row_base = wave_m * (next.half ? kWaveRows / 2 : kWaveRows);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            lhs_frag0[q] = fragment_base<kLhsContiguousK>(wave_row_base, q, lane);
+            lhs_frag[q] = lhs_frag0[q] + lhs_now;
+            lhs_frag_next[q] = lhs_frag0[q] + lhs_next;
+            rhs_frag[q] = fragment_base<kRhsContiguousK>(wave_n * kWaveCols, q, lane);
+        }
+    };
+    auto continue_tile = [&]() {
         load_lhs.advance();
         load_rhs.advance();
 #pragma unroll
@@ -989,60 +1110,88 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         load_lhs.advance();
 #pragma unroll
         for (int j = 0; j < 2; ++j) load_lhs.load(lhs_after, j);
-        clear_accumulators();  // 256 register writes, while the first loads are on their way
-        wait_for_loads<14>();  // 30 loads so far, the first 16 of them slice 0
-        __syncthreads();
-        mask_slice(0, lhs_now, 0);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            read_rhs_fragment(0, 0, 0, q);
-            read_lhs_fragment(false, 0, 0, q);
-        }
-        constexpr std::integral_constant<int, 0> slot0{};
-        constexpr std::integral_constant<int, 1> slot1{};
-        // Two slices per trip (the rhs slots alternate); an odd count multiplies one slice of zeros. (Leaving the
-        // loop before that slice costs far more than it saves: with a second exit the compiler no longer keeps the
-        // accumulators in place and the kernel ran five times slower.)
-        if (half_tile) {
-            for (int t = 0; t < num_slices; t += 2) {
-                iteration(t, slot0, std::true_type{});
-                iteration(t + 1, slot1, std::true_type{});
-            }
-        } else {
-            for (int t = 0; t < num_slices; t += 2) {
-                iteration(t, slot0, std::false_type{});
-                iteration(t + 1, slot1, std::false_type{});
-            }
-        }
-        wait_for_loads<0>();  // the zero-filling loads of slices past the end still write LDS
-    } else {
-        clear_accumulators();
-    }
+    };
 
-    if (piece_slot < 0 && args.accumulate != 0 && num_slices == 0) return;  // nothing to add
-    __syncthreads();  // all wavefronts are done reading operand slices; LDS becomes the staging area
-    if constexpr (kFusion == kFusionGatedForward) {
-        T *layer_1 = args.out == nullptr ? nullptr : static_cast<T *>(args.out) + work.out_offset;
-        FM_DISPATCH_ACTIVATION(args.activation, kActivation,
-                               store_tile_gated_forward<T, kActivation>(
-                                   acc, lds, layer_1, static_cast<T *>(args.fused_out) + work.fused_offset,
-                                   args.out_stride_row, args.fused_stride, args.half, work.rows_valid, wave, lane));
-    } else if constexpr (kFusion == kFusionGatedBackward) {
-        T *recomputed = args.fused_out == nullptr ? nullptr : static_cast<T *>(args.fused_out) + work.fused_offset;
-        FM_DISPATCH_ACTIVATION(args.activation, kActivation,
-                               store_tile_gated_backward<T, kActivation>(
-                                   acc, lds, static_cast<T *>(args.out) + work.out_offset,
-                                   static_cast<const T *>(args.fused_in) + work.out_offset, recomputed,
-                                   args.out_stride_row, args.fused_stride, args.half, work.rows_valid, work.cols_valid,
-                                   wave, lane));
-    } else {
-        if (piece_slot >= 0)
-            store_partial(acc, args.partials + static_cast<int64_t>(piece_slot) * kPartialFloats, wave, lane);
-        else
-            store_result(
-                args, work, [&](int i) -> const f32x16_t(&)[kTilesN] { return acc[i]; }, lds, wave, lane, wave_row_base,
-                wave_row_blocks);
+    first_loads(tile);
+    while (true) {
+        setup_tile(tile);
+        const int num_slices = tile.num_slices;
+        if (num_slices > 0) {
+            // Prologue: slice 0, lhs slice 1 and the first pieces of the slices after them on their way; slice 0 landed.
+            continue_tile();
+            clear_accumulators();  // 256 register writes, while the first loads are on their way
+            wait_for_loads<14>();  // 30 loads since the tile began, the first 16 of them slice 0
+            __syncthreads();
+            mask_slice(0, lhs_now, 0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                read_rhs_fragment(0, 0, 0, q);
+                read_lhs_fragment(false, 0, 0, q);
+            }
+            constexpr std::integral_constant<int, 0> slot0{};
+            constexpr std::integral_constant<int, 1> slot1{};
+            // Two slices per trip (the rhs slots alternate); an odd count multiplies one slice of zeros. (Leaving the
+            // loop before that slice costs far more than it saves: with a second exit the compiler no longer keeps the
+            // accumulators in place and the kernel ran five times slower.)
+            if (tile.half) {
+                for (int t = 0; t < num_slices; t += 2) {
+                    iteration(t, slot0, std::true_type{});
+                    iteration(t + 1, slot1, std::true_type{});
+                }
+            } else {
+                for (int t = 0; t < num_slices; t += 2) {
+                    iteration(t, slot0, std::false_type{});
+                    iteration(t + 1, slot1, std::false_type{});
+                }
+            }
+            wait_for_loads<0>();  // the zero-filling loads of slices past the end still write LDS
+        } else {
+            clear_accumulators();
+        }
+        __syncthreads();  // all wavefronts are done reading operand slices; LDS becomes the staging area
+        forget_arguments();
+
+        // What the epilogue needs of this tile, before the next one takes its place.
+        const TileRecord work = tile.work;
+        const int piece_slot = tile.piece_slot;
+        const int wave_row_base = wave_m * (tile.half ? kWaveRows / 2 : kWaveRows);
+        const int wave_row_blocks = tile.half ? kTilesM / 2 : kTilesM;
+        // The next tile is looked up here, not earlier, to keep its coordinates out of the registers of the main loop;
+        // its first loads go out before this tile's results do.
+        id += gridDim.x;
+        const bool have_next = id < args.num_ids && find_tile(id, tile);
+        if (have_next) first_loads(tile);
+
+        FM_LDS(char) *staging = lds + kStagingBase;
+        const int lane = opaque(static_cast<int>(threadIdx.x & 63));  // per-lane addresses of the epilogue: not hoisted
+        if (piece_slot < 0 && args.accumulate != 0 && num_slices == 0) {
+            // nothing to add
+        } else if constexpr (kFusion == kFusionGatedForward) {
+            T *layer_1 = args.out == nullptr ? nullptr : static_cast<T *>(args.out) + work.out_offset;
+            FM_DISPATCH_ACTIVATION(args.activation, kActivation,
+                                   store_tile_gated_forward<T, kActivation>(
+                                       acc, staging, layer_1, static_cast<T *>(args.fused_out) + work.fused_offset,
+                                       args.out_stride_row, args.fused_stride, args.half, work.rows_valid, wave, lane));
+        } else if constexpr (kFusion == kFusionGatedBackward) {
+            T *recomputed = args.fused_out == nullptr ? nullptr : static_cast<T *>(args.fused_out) + work.fused_offset;
+            FM_DISPATCH_ACTIVATION(args.activation, kActivation,
+                                   store_tile_gated_backward<T, kActivation>(
+                                       acc, staging, static_cast<T *>(args.out) + work.out_offset,
+                                       static_cast<const T *>(args.fused_in) + work.out_offset, recomputed,
+                                       args.out_stride_row, args.fused_stride, args.half, work.rows_valid,
+                                       work.cols_valid, wave, lane));
+        } else {
+            if (piece_slot >= 0)
+                store_partial(acc, args.partials + static_cast<int64_t>(piece_slot) * kPartialFloats, wave, lane);
+            else
+                store_result(
+                    args, work, [&](int i) -> const f32x16_t(&)[kTilesN] { return acc[i]; }, staging, wave, lane,
+                    wave_row_base, wave_row_blocks);
+        }
+        if (!have_next) break;
+        __syncthreads();  // the staging areas have been read: the next tile's loads may overwrite them
     }
+#undef args
 }
 
 // Adds the pieces of each tile whose reduction the main kernel split, in piece order, and stores the sums.
@@ -1108,11 +1257,11 @@ static int launch_instance(const GemmArgs &args, hipStream_t stream) {
     auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK, kMasked, kFusion>;
     static std::atomic<uint64_t> configured{0};
     if (int status = allow_lds(reinterpret_cast<const void *>(kernel), kLdsBytes, configured)) return status;
-    // Whole rounds of one chunk per XCD; the surplus workgroups find no tile and exit. With a workspace the pieces
-    // of the last round's tiles come after the whole tiles, at most kMaxPartials of them.
-    int grid = (args.tiles_m * args.tiles_n + kRound - 1) / kRound * kRound;
-    if (args.partials != nullptr) grid += kMaxPartials;
-    kernel<<<grid, kMfmaThreads, kLdsBytes, stream>>>(args);
+    // With a workspace, one wavefront per id first writes the id's tile record.
+    if (args.tile_table != nullptr)
+        grouped_gemm_plan_kernel<<<(args.num_ids + 3) / 4, 256, 0, stream>>>(args, static_cast<TileRecord *>(args.tile_table));
+    // One workgroup per CU walks the ids (see the kernel).
+    kernel<<<min(args.num_ids, kRound), kMfmaThreads, kLdsBytes, stream>>>(args);
     if (args.partials != nullptr) {
         static std::atomic<uint64_t> reduce_configured{0};
         if (int status = allow_lds(reinterpret_cast<const void *>(grouped_gemm_reduce_kernel), kReduceLdsBytes,
@@ -1176,19 +1325,24 @@ bool mfma_gemm_fusion_eligible(const GemmArgs &args, int dtype) {
     return true;
 }
 
-// ---- workspace for split reductions --------------------------------------------------------------------
+// ---- workspace: the tile table and the pieces of split reductions ----------------------------------------
 // Whether a product is one whose last round is split is decided from its dimensions alone (few rounds of long tiles);
-// the caller then brings kMaxPartials tile-sized fp32 slots. Given the dimensions, whether the split happens depends
-// on nothing but the presence of the workspace, which is the caller's choice.
+// the caller then brings kMaxPartials tile-sized fp32 slots, followed by one tile record per workgroup id. Given the
+// dimensions, whether the split happens depends on nothing but the presence of the workspace, which is the caller's
+// choice; the table changes no result, only where a workgroup finds its tile.
 static void count_tiles(GemmArgs &args) {
     if (args.mode == kInputRowSparse) {
         args.tiles_m = static_cast<int>((args.sparse_size + kTile - 1) / kTile) * args.num_experts;
     } else {
-        // Upper bound of sum_e ceil(rows_e / 256); surplus workgroups find no tile and exit.
+        // Upper bound of sum_e ceil(rows_e / 256); the surplus ids have no tile.
         args.tiles_m = static_cast<int>((args.rows + kTile - 1) / kTile + (args.num_experts > 1 ? args.num_experts : 0));
     }
     args.tiles_n = static_cast<int>((args.cols + kTile - 1) / kTile);
     if (args.fusion == kFusionGatedForward) args.tiles_n = static_cast<int>(args.half / (kTile / 2));
+}
+
+static bool too_many_tiles(const GemmArgs &args) {
+    return static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31) - 2 * kRound - kMaxPartials;
 }
 
 static bool splits_last_round(const GemmArgs &args) {
@@ -1197,24 +1351,38 @@ static bool splits_last_round(const GemmArgs &args) {
            static_cast<int64_t>(args.tiles_m) * args.tiles_n <= kMaxRoundsToSplit * kRound;
 }
 
+// Whole rounds of one chunk per XCD; when the last round is split its pieces come after the whole tiles, at most
+// kMaxPartials of them.
+static int count_ids(const GemmArgs &args, bool split) {
+    return (args.tiles_m * args.tiles_n + kRound - 1) / kRound * kRound + (split ? kMaxPartials : 0);
+}
+
+constexpr size_t kPartialBytes = sizeof(float) * kPartialFloats * kMaxPartials;
+static size_t table_bytes(int num_ids) { return (static_cast<size_t>(num_ids) * sizeof(TileRecord) + 255) / 256 * 256; }
+
 size_t mfma_gemm_workspace_size(GemmArgs args) {
     if (args.rows <= 0 || args.cols <= 0 || args.inner <= 0) return 0;
     count_tiles(args);
-    return splits_last_round(args) ? sizeof(float) * kPartialFloats * kMaxPartials : 0;
+    if (too_many_tiles(args)) return 0;
+    const bool split = splits_last_round(args);
+    return (split ? kPartialBytes : 0) + table_bytes(count_ids(args, split));
 }
 
 int mfma_gemm_launch(GemmArgs args, int dtype, void *workspace, size_t workspace_size, hipStream_t stream) {
     count_tiles(args);
-    if (static_cast<int64_t>(args.tiles_m) * args.tiles_n >= (int64_t(1) << 31) - 1024)
-        return fail(FM_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
+    if (too_many_tiles(args)) return fail(FM_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
     args.partials = nullptr;
-    if (workspace != nullptr && splits_last_round(args)) {
-        const size_t needed = sizeof(float) * kPartialFloats * kMaxPartials;
-        if (workspace_size < needed || !aligned16(workspace))
+    args.tile_table = nullptr;
+    const bool split = workspace != nullptr && splits_last_round(args);
+    args.num_ids = count_ids(args, split);
+    if (workspace != nullptr) {
+        const size_t needed = (split ? kPartialBytes : 0) + table_bytes(args.num_ids);
+        if (workspace_size < needed || reinterpret_cast<uintptr_t>(workspace) % 64 != 0)
             return fail(FM_ERR_INVALID_ARGUMENT,
-                        "grouped gemm: workspace of %zu bytes (16-byte aligned) needed, got %zu at %p", needed,
+                        "grouped gemm: workspace of %zu bytes (64-byte aligned) needed, got %zu at %p", needed,
                         workspace_size, workspace);
-        args.partials = static_cast<float *>(workspace);
+        if (split) args.partials = static_cast<float *>(workspace);
+        args.tile_table = static_cast<char *>(workspace) + (split ? kPartialBytes : 0);
     }
     return dtype == FM_DTYPE_BF16 ? launch_layout<bf16_t>(args, stream) : launch_layout<f16_t>(args, stream);
 }

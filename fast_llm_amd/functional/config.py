@@ -25,11 +25,13 @@ class KernelConfig:
     # same arithmetic at full occupancy behind its memory traffic. It pays only where layer 1's output is not
     # stored at all (inference, full recomputation: 3.27 ms against 3.14 + 0.24 ms).
     fuse_activation = False
-    # Hand the grouped products the scratch with which a launch of few, long tiles (layer 2 forward and the layer 1
-    # input gradient at the Mixtral shape: 4.1 rounds of tiles on 256 CUs) cuts the reductions of its last round's
-    # tiles into pieces that fill the idle CUs. Split and unsplit sums differ in the last bits; with a fixed setting
-    # results are reproducible whatever the stream or allocator state.
-    split_last_round = True
+    # Hand the grouped products their scratch: a table of where every tile of a launch lies, written by a small
+    # kernel before the product (the product's workgroups then look their tiles up instead of each scanning the expert
+    # map), and the space with which a launch of few, long tiles (layer 2 forward and the layer 1 input gradient at
+    # the Mixtral shape: 4.1 rounds of tiles on 256 CUs) cuts the reductions of its last round's tiles into pieces
+    # that fill the idle CUs. Split and unsplit sums differ in the last bits; with a fixed setting results are
+    # reproducible whatever the stream or allocator state.
+    grouped_gemm_workspace = True
 
     @classmethod
     def enabled(cls, device: "torch.device|None" = None, default: bool | None = None) -> bool:

@@ -43,12 +43,17 @@ def _launch(
     pointers = [_lib.ptr(lhs.detach()), _lib.ptr(rhs.detach()), _lib.ptr(out), _lib.ptr(expert_ends)]
     if with_pad_begins:
         pointers.append(_lib.ptr(expert_pad_begins))
-    # Scratch for splitting the last round of a launch with few, long tiles. A torch allocation per call: the caching
-    # allocator hands the same block back to calls on one stream and keeps calls on different streams apart, also
-    # under graph capture. Whether a product splits depends on its dimensions and this switch only.
+    # Scratch for the tile table and for splitting the last round of a launch with few, long tiles. A torch allocation
+    # per call: the caching allocator hands the same block back to calls on one stream and keeps calls on different
+    # streams apart, also under graph capture. Whether a product splits depends on its dimensions and this switch only.
     workspace, workspace_size = None, 0
-    if KernelConfig.split_last_round and not with_pad_begins:
-        workspace_size = _lib.lib().fm_grouped_gemm_workspace_size(*dims, num_experts, _lib.dtype_tag(lhs.dtype))
+    if KernelConfig.grouped_gemm_workspace:
+        size_function = (
+            _lib.lib().fm_input_row_sparse_matmul_workspace_size
+            if with_pad_begins
+            else _lib.lib().fm_grouped_gemm_workspace_size
+        )
+        workspace_size = size_function(*dims, num_experts, _lib.dtype_tag(lhs.dtype))
         if workspace_size:
             workspace = torch.empty(workspace_size, dtype=torch.uint8, device=device)
     _lib.call(

@@ -242,20 +242,29 @@ int fm_mlp_activation_backward(const void *grad_output, void *grad_input, const 
  * Results are deterministic (no floating-point atomics; every sum has a fixed order that depends only on the
  * arguments and the expert map).
  *
- * `workspace`: a launch of few, long tiles (at most 16 rounds of 256 tiles of 256 x 256, reduction of 2048 or more)
- * leaves most CUs idle in its last round; given `fm_grouped_gemm_workspace_size(...)` bytes of device scratch
- * (16-byte aligned, content irrelevant) the output-sparse and input-inner-sparse products cut the reductions of that
- * round's tiles into 2, 4 or 8 pieces that fill the CUs and add the pieces in piece order. Whether this happens
- * depends on the dimensions and on whether a workspace is passed, on nothing else (not on the stream, the device's
- * free memory or earlier calls): NULL with size 0 selects the unsplit sums, which differ from the split ones in
- * the last bits; a non-null workspace smaller than required is FM_ERR_INVALID_ARGUMENT. Calls that may overlap
- * (different streams) need different workspaces. The row-sparse product never splits and ignores the pair.
+ * `workspace`: device scratch (64-byte aligned, content irrelevant) of `fm_grouped_gemm_workspace_size(...)` bytes
+ * (`fm_input_row_sparse_matmul_workspace_size(...)` for the row-sparse product). With it, a small kernel first writes
+ * where every tile of the launch lies, so that the workgroups of the product look their tiles up instead of each
+ * scanning the expert map (same tiles, same results); and a launch of few, long tiles (at most 16 rounds of 256
+ * tiles of 256 x 256, reduction of 2048 or more) of the output-sparse and input-inner-sparse products, which would
+ * leave most CUs idle in its last round, cuts the reductions of that round's tiles into 2, 4 or 8 pieces that fill
+ * the CUs and adds the pieces in piece order. Whether that split happens depends on the dimensions and on whether a
+ * workspace is passed, on nothing else (not on the stream, the device's free memory or earlier calls): NULL with
+ * size 0 selects the unsplit sums, which differ from the split ones in the last bits; a non-null workspace smaller
+ * than required or misaligned is FM_ERR_INVALID_ARGUMENT. Calls that may overlap (different streams) need different
+ * workspaces. Products that do not run on the matrix cores (fp32 operands, odd strides) ignore the pair.
  * --------------------------------------------------------------------------------------------------------- */
 
-/* Bytes of workspace with which a product `out [row_dim, col_dim] = lhs [row_dim, inner_dim] x rhs` of `dtype`
- * operands over `num_experts` experts (1 for a dense product) splits its last round; 0 if it never splits. */
+/* Bytes of workspace for a product `out [row_dim, col_dim] = lhs [row_dim, inner_dim] x rhs` of `dtype` operands over
+ * `num_experts` experts (1 for a dense product): the tile table and, where the last round is split, its pieces.
+ * 0 for fp32 operands or an empty product. Depends on these five numbers only. */
 size_t fm_grouped_gemm_workspace_size(int64_t row_dim, int64_t col_dim, int64_t inner_dim, int64_t num_experts,
                                       int dtype);
+
+/* The same for the row-sparse product `out [row_sparse_dim * num_experts, col_dim]` (its reductions are never split:
+ * the tile table only). */
+size_t fm_input_row_sparse_matmul_workspace_size(int64_t row_sparse_dim, int64_t col_dim, int64_t inner_dim,
+                                                 int64_t num_experts, int dtype);
 
 /* out[i, j] = sum_k lhs[i, k] * rhs[k, j + col_sparse_dim * e(i)]   for i < expert_ends[-1]; rows past the last
  * expert ("phantom" rows) are neither read nor written. Padding rows inside an expert are computed like

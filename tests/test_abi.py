@@ -65,14 +65,24 @@ def test_argument_validation_returns_status_and_message(library):
 
 
 def test_grouped_gemm_workspace_size_depends_on_the_dimensions_only(library):
-    # Layer 2 forward at the Mixtral shape: 66 + 8 row tiles x 16 column tiles, reduction 14336 -> splits.
+    partials = 512 * 256 * 256 * 4  # the pieces of a split last round
+    record = 64  # bytes of the tile table per workgroup id
+
+    def ids(row_tiles, column_tiles, split):  # whole rounds of 256 ids, then the pieces
+        return -(-row_tiles * column_tiles // 256) * 256 + (512 if split else 0)
+
+    # Layer 2 forward at the Mixtral shape: 68 + 8 row tiles x 16 column tiles, reduction 14336 -> splits.
     size = library.fm_grouped_gemm_workspace_size(17408, 4096, 14336, 8, 1)
-    assert size == 512 * 256 * 256 * 4
+    assert size == partials + ids(76, 16, True) * record
     assert library.fm_grouped_gemm_workspace_size(17408, 4096, 14336, 8, 2) == size
     assert library.fm_grouped_gemm_workspace_size(17408, 4096, 14336, 8, 0) == 0  # fp32: generic kernel
-    assert library.fm_grouped_gemm_workspace_size(17408, 28672, 4096, 8, 1) == 0  # layer 1 forward: 29 rounds
-    assert library.fm_grouped_gemm_workspace_size(17408, 4096, 1984, 8, 1) == 0  # short reduction
+    # Layer 1 forward (29 rounds) and a short reduction are not split: the table only.
+    assert library.fm_grouped_gemm_workspace_size(17408, 28672, 4096, 8, 1) == ids(76, 112, False) * record
+    assert library.fm_grouped_gemm_workspace_size(17408, 4096, 1984, 8, 1) == ids(76, 16, False) * record
     assert library.fm_grouped_gemm_workspace_size(0, 4096, 14336, 8, 1) == 0
+    # The row-sparse product never splits: 8 experts x 56 row tiles x 16 column tiles.
+    assert library.fm_input_row_sparse_matmul_workspace_size(14336, 4096, 17408, 8, 1) == ids(8 * 56, 16, False) * record
+    assert library.fm_input_row_sparse_matmul_workspace_size(14336, 4096, 17408, 8, 0) == 0
 
 
 def test_router_and_fused_entry_points_validate_before_launching(library):

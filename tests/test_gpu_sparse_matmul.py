@@ -361,9 +361,11 @@ def test_split_does_not_depend_on_stream_or_history(device, library):
     rows = oracle_map.num_rows
     generator = torch.Generator().manual_seed(21)
     x, weight = _normal(rows, inner, dtype, generator).to(device), _normal(experts * other, inner, dtype, generator).to(device)
-    assert library.fm_grouped_gemm_workspace_size(rows, other, inner, experts, _lib.dtype_tag(dtype)) > 0
+    split_size = library.fm_grouped_gemm_workspace_size(rows, other, inner, experts, _lib.dtype_tag(dtype))
+    assert split_size > 128 << 20  # 512 partial tiles of 256 x 256 floats, then the tile table
     assert library.fm_grouped_gemm_workspace_size(rows, other, inner, experts, _lib.dtype_tag(torch.float32)) == 0
-    assert library.fm_grouped_gemm_workspace_size(rows, other, 1024, experts, _lib.dtype_tag(dtype)) == 0
+    # A short reduction is not split: the tile table only.
+    assert 0 < library.fm_grouped_gemm_workspace_size(rows, other, 1024, experts, _lib.dtype_tag(dtype)) < 1 << 20
 
     def product():
         return output_sparse_matmul(x, weight.t(), sparse_map)
@@ -389,12 +391,12 @@ def test_split_does_not_depend_on_stream_or_history(device, library):
         assert torch.equal(captured, expected)
         assert torch.equal(product(), expected)  # eager work between the replays
 
-    KernelConfig.split_last_round = False
+    KernelConfig.grouped_gemm_workspace = False
     try:
         unsplit = product()
         assert torch.equal(product(), unsplit)
     finally:
-        KernelConfig.split_last_round = True
+        KernelConfig.grouped_gemm_workspace = True
     assert not torch.equal(unsplit, expected)  # another order of the same sums
     assert max_rel_err(unsplit.cpu(), expected.cpu()) <= _MAX_REL[dtype]
 
@@ -408,6 +410,44 @@ def test_split_does_not_depend_on_stream_or_history(device, library):
         _lib.index_tag(torch.int32), small.data_ptr(), size - 1, torch.cuda.current_stream(device).cuda_stream,
     )  # fmt: skip
     assert status == _lib.FM_ERR_INVALID_ARGUMENT and b"workspace" in library.fm_last_error()
+
+
+def test_tile_table_changes_no_bit(device):
+    """With a workspace the workgroups read where their tiles lie from a table written by a small kernel, without one
+    each scans the expert map itself: the same tiles either way, so products that are not split are bit-identical
+    (ragged experts with half tiles, an empty expert, all three products, accumulation into fp32)."""
+    from fast_llm_amd.functional.config import KernelConfig
+
+    experts, inner, other, dtype = 7, 192, 328, torch.bfloat16
+    case = _ragged_case(1500, experts)
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device, torch.int32)
+    rows = oracle_map.num_rows
+    generator = torch.Generator().manual_seed(5)
+    x = _normal(rows, inner, dtype, generator).to(device)
+    y = _normal(rows, other, dtype, generator).to(device)
+    weight = _normal(experts * other, inner, dtype, generator).to(device)
+    previous = torch.randn(experts * other, inner, generator=generator).to(device)
+
+    def products():
+        return (
+            output_sparse_matmul(x, weight.t(), sparse_map),
+            input_inner_sparse_matmul(y, weight, sparse_map),
+            input_row_sparse_matmul(y.t(), x, sparse_map),
+            input_row_sparse_matmul(y.t(), x, sparse_map, out=previous.clone(), accumulate=True),
+        )
+
+    with_table = products()
+    KernelConfig.grouped_gemm_workspace = False
+    try:
+        without = products()
+    finally:
+        KernelConfig.grouped_gemm_workspace = True
+    valid = sparse_map.expert_ends[-1].item()
+    for a, b in zip(with_table[:2], without[:2]):
+        assert torch.equal(a[:valid], b[:valid])
+    for a, b in zip(with_table[2:], without[2:]):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("seed", range(24))
