@@ -158,7 +158,9 @@ __global__ __launch_bounds__(kCopyThreads) void copy_sparse_to_dense_kernel(cons
 // grad_scores[t, j] = <input[row(t, j), :], grad_output[t, :]>; when kFused also
 // grad_input[row(t, j), :] = grad_output[t, :] * scores[t, j].
 // kChunks vectors of grad_output per lane are kept in registers across the k slots.
-template <typename T, typename OutT, bool kVector, bool kFused, int kChunks, bool kStreamGather = false>
+// kAhead: the rows of slot j + 1 are requested before slot j is reduced (pays from three slots per token on).
+template <typename T, typename OutT, bool kVector, bool kFused, int kChunks, bool kStreamGather = false,
+          bool kAhead = false>
 __global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__restrict__ input,
                                                                   const T *__restrict__ grad_output,
                                                                   T *__restrict__ grad_input,
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__res
         }
     };
 
-    if constexpr (kChunks > 0) {
+    if constexpr (kChunks > 0 && kAhead) {
         // The lane's vectors of slot j + 1 are requested before slot j is reduced (two barriers and an LDS round trip
         // per slot): a slot's memory latency overlaps the previous slot's reduction.
         struct Slot {
@@ -262,17 +264,26 @@ __global__ __launch_bounds__(kCopyThreads) void grad_score_kernel(const T *__res
             if (row >= 0 && row < args.num_rows_sparse) {
                 const T *in_row = input + row * columns;
                 T *out_row = kFused ? grad_input + row * columns : nullptr;
-                for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns;
-                     c += static_cast<int64_t>(blockDim.x) * N) {
-                    Vec16<T> g, value;
-                    if constexpr (kVector) {
-                        g = load16(grad_row + c);
-                        value = load16(in_row + c);
-                    } else {
-                        g.v[0] = grad_row[c];
-                        value.v[0] = in_row[c];
-                    }
+                auto column = [&](const Vec16<T> &g, int64_t c) {
+                    Vec16<T> value;
+                    if constexpr (kVector) value = kStreamGather ? load16_stream(in_row + c) : load16(in_row + c);
+                    else value.v[0] = in_row[c];
                     products(value, g, score, out_row + c, partial);
+                };
+                if constexpr (kChunks > 0) {
+#pragma unroll
+                    for (int q = 0; q < kChunks; ++q) {
+                        const int64_t c = (static_cast<int64_t>(q) * blockDim.x + threadIdx.x) * N;
+                        if (c < columns) column(grad[q], c);
+                    }
+                } else {
+                    for (int64_t c = static_cast<int64_t>(threadIdx.x) * N; c < columns;
+                         c += static_cast<int64_t>(blockDim.x) * N) {
+                        Vec16<T> g;
+                        if constexpr (kVector) g = load16(grad_row + c);
+                        else g.v[0] = grad_row[c];
+                        column(g, c);
+                    }
                 }
             }
             finish_slot(j, partial);
@@ -405,12 +416,17 @@ static void launch_grad_score(const void *input, const void *grad_output, void *
     const int vector = vectorised ? Vec16<T>::N : 1;
     const int64_t chunks = (args.num_columns + static_cast<int64_t>(vector) * threads - 1) /
                            (static_cast<int64_t>(vector) * threads);
-#define FM_LAUNCH_GS(VEC, CHUNKS)                                                                                   \
+#define FM_LAUNCH_GS_STREAM(VEC, CHUNKS, STREAM)                                                                   \
     do {                                                                                                            \
-        if (args.stream_gather && CHUNKS > 0)                                                                       \
-            grad_score_kernel<T, OutT, VEC, kFused, CHUNKS, true><<<rows, threads, 0, stream>>>(in, go, gi, gs, args); \
+        if (args.experts_per_token > 2 && CHUNKS > 0)                                                               \
+            grad_score_kernel<T, OutT, VEC, kFused, CHUNKS, STREAM, true><<<rows, threads, 0, stream>>>(in, go, gi, gs, args); \
         else                                                                                                        \
-            grad_score_kernel<T, OutT, VEC, kFused, CHUNKS, false><<<rows, threads, 0, stream>>>(in, go, gi, gs, args); \
+            grad_score_kernel<T, OutT, VEC, kFused, CHUNKS, STREAM, false><<<rows, threads, 0, stream>>>(in, go, gi, gs, args); \
+    } while (0)
+#define FM_LAUNCH_GS(VEC, CHUNKS)                                       \
+    do {                                                                \
+        if (args.stream_gather) FM_LAUNCH_GS_STREAM(VEC, CHUNKS, true); \
+        else FM_LAUNCH_GS_STREAM(VEC, CHUNKS, false);                   \
     } while (0)
     if (vectorised) {
         if (chunks <= 1) FM_LAUNCH_GS(true, 1);
@@ -421,6 +437,7 @@ static void launch_grad_score(const void *input, const void *grad_output, void *
         FM_LAUNCH_GS(false, 0);
     }
 #undef FM_LAUNCH_GS
+#undef FM_LAUNCH_GS_STREAM
 }
 
 template <bool kFused>
