@@ -159,6 +159,8 @@ struct TileLoader {
     uint32_t num_records;    // wave-uniform: lane offsets >= this bring zeros
     int64_t step;            // bytes from one slice to the next
     int slices_left;         // slices after the one being fetched
+    uint32_t last_records;   // row-contiguous: `num_records` of the last slice (its K-rows past the reduction range
+                             // bring zeros)
     int lds_offset;          // wave-uniform: of this wavefront's first 1 KiB block within an operand slot
 
     // `stride`: bytes between rows (K-contiguous) or between K-rows (row-contiguous). Rows >= valid_rows are never
@@ -167,8 +169,10 @@ struct TileLoader {
     // `split_rows` (K-contiguous only, 0: off): rows 64..127 and 192..255 of the tile are not the rows after 0..63 and
     // 128..191 but lie `split_rows` rows after them, i.e. tile row n is memory row
     // (n / 128) * 64 + n % 64 + (n / 64 % 2) * split_rows (the gate and up halves of a gated layer's weight).
+    // `k_count`: reduction indices from the first one of slice 0 to the end of the reduction range; a row-contiguous
+    // operand gets zeros for the K-rows of its last slice that lie past it.
     __device__ __forceinline__ void setup(const char *tile_base, int64_t stride, int valid_rows, int num_slices,
-                                          int wave, int lane, int split_rows = 0) {
+                                          int k_count, int wave, int lane, int split_rows = 0) {
         static_assert(kLoadsPerOperand % 2 == 0, "loads come in (even, odd) pairs");
         fetch_base = tile_base;
         slices_left = num_slices - 1;
@@ -193,8 +197,13 @@ struct TileLoader {
         // Two loads further on: 128 slots = 16 rows of a K-contiguous slice, 4 K-rows of a row-contiguous one.
         pair_stride = static_cast<uint32_t>((kContiguousK ? 128 / kChunksPerRow : 4) * stride);
         const int64_t last_row = split_rows == 0 ? valid_rows - 1 : split_rows + kTile / 2 - 1;
-        num_records = kContiguousK ? static_cast<uint32_t>(last_row * stride + kBK * 2) : 0xffffffffu;
         step = kContiguousK ? kBK * 2 : kBK * stride;
+        if constexpr (kContiguousK) {
+            num_records = last_records = static_cast<uint32_t>(last_row * stride + kBK * 2);
+        } else {
+            last_records = static_cast<uint32_t>((k_count - (num_slices - 1) * kBK) * stride);
+            num_records = num_slices == 1 ? last_records : 0xffffffffu;
+        }
     }
 
     // Move on to the next slice. Past the last slice the descriptor's range becomes empty, so that every further
@@ -203,7 +212,7 @@ struct TileLoader {
         // Said to be wave-uniform once more: loop-carried values otherwise end up in vector registers.
         fetch_base = uniform_pointer(fetch_base + step);
         slices_left = __builtin_amdgcn_readfirstlane(slices_left - 1);
-        num_records = __builtin_amdgcn_readfirstlane(slices_left < 0 ? 0u : num_records);
+        num_records = __builtin_amdgcn_readfirstlane(slices_left < 0 ? 0u : (slices_left == 0 ? last_records : num_records));
     }
 
     // Chunk j of the slice being fetched -> the operand slot that starts at LDS byte address `slot_address`.
@@ -898,10 +907,11 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     // would hand that CU if all tiles took the same time, and the first loads of a tile are issued before the
     // previous tile is written out. Ids map to tiles in increasing order, so the first id without a tile ends the walk.
     // Everything about a tile is the same in every lane and is said to be, so that it lives in scalar registers.
+    constexpr bool kSlicesFromRangeStart = kMasked && !kLhsContiguousK && !kRhsContiguousK;
     struct Tile {
         TileRecord work;
         int piece_slot;   // >= 0: a piece of a split reduction, stored to that workspace slot
-        int k_first;      // first reduction index of slice 0 (a multiple of kBK)
+        int k_first;      // first reduction index of slice 0
         int num_slices;
         bool half;        // at most 128 valid rows: the wavefronts share them, 64 each, and issue half the MFMAs
     };
@@ -919,8 +929,10 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         }
         const TileRecord &work = tile.work;
         tile.piece_slot = work.piece_slot;
-        tile.k_first = work.k_lo / kBK * kBK;
-        const int k_last = work.k_hi > work.k_lo ? (work.k_hi + kBK - 1) / kBK * kBK : tile.k_first;
+        // Slices start at multiples of kBK, except where both operands are row-contiguous (any K-row can start a
+        // slice then): the ragged range of the row-sparse product starts with its first slice and needs no masking.
+        tile.k_first = kSlicesFromRangeStart ? work.k_lo : work.k_lo / kBK * kBK;
+        const int k_last = work.k_hi > work.k_lo ? tile.k_first + (work.k_hi - tile.k_first + kBK - 1) / kBK * kBK : tile.k_first;
         tile.num_slices = (k_last - tile.k_first) / kBK;
         // A tile with at most 128 valid rows (the last row tile of an expert whose padded row count is an odd multiple
         // of 128) is a half tile. The transfers stay as they are (the rows past the valid ones bring zeros or repeats
@@ -977,7 +989,7 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
                                        : load_fragment<kLhsContiguousK>(lds, lhs_frag, 0, i, kstep);
     };
     auto mask_slice = [&](int slice, int lhs_address, int rhs_slot) {
-        if constexpr (kMasked) {
+        if constexpr (kMasked && !kSlicesFromRangeStart) {
             const int k_lo = tile.work.k_lo, k_hi = tile.work.k_hi;
             const int k0 = tile.k_first + slice * kBK;
             if (slice < tile.num_slices && (k0 < k_lo || k0 + kBK > k_hi)) {  // wave-uniform
@@ -1069,10 +1081,11 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
                           (work.rhs_offset + next.k_first * args.rhs_stride_inner) * static_cast<int64_t>(sizeof(T));
         lhs_loader.setup(uniform_pointer(lhs),
                          (kLhsContiguousK ? args.lhs_stride_row : args.lhs_stride_inner) * sizeof(T), work.rows_valid,
-                         next.num_slices, wave, lane);
+                         next.num_slices, work.k_hi - next.k_first, wave, lane);
         rhs_loader.setup(uniform_pointer(rhs),
                          (kRhsContiguousK ? args.rhs_stride_col : args.rhs_stride_inner) * sizeof(T), work.cols_valid,
-                         next.num_slices, wave, lane, kFusion == kFusionGatedForward ? static_cast<int>(args.half) : 0);
+                         next.num_slices, work.k_hi - next.k_first, wave, lane,
+                         kFusion == kFusionGatedForward ? static_cast<int>(args.half) : 0);
     };
     constexpr int kFirstLhsSlot = kLhsBase + (kLhsStages - 1) * kOperandBytes;
     auto first_loads = [&](const Tile &next) {
