@@ -7,11 +7,12 @@
 //                        token axis, everything outside replaced by zero before the multiply
 // (reference semantics: fast_llm/functional/triton/sparse_linear.py:185-258, 310-385, 437-517).
 //
-// Half-precision operands with vectorisable layouts go to the MFMA kernel (fm_gemm_mfma.hip). Everything else
-// (fp32 operands, odd strides or sizes) goes to the generic kernel below: a 64 x 64 x 16 LDS-tiled kernel with
-// full bounds checks and true fp32 multiply-adds, which is also what the 1e-5 fp32 parity bound needs. The
-// generic kernel computes a 64-row block that straddles an expert boundary in one pass per expert, so it takes any
-// padding multiple.
+// Half-precision operands with vectorisable layouts go to the MFMA kernel (fm_gemm_mfma.hip). fp32 operands go to
+// the fp32 matrix-core kernel below (128 x 128 x 16 tiles of v_mfma_f32_32x32x2_f32: true fp32 multiply-adds, which
+// is what the 1e-5 fp32 parity bound needs; 59-63 TFLOP/s at 16384 x 4096 x 2048 over 8 experts). Everything else
+// (half-precision operands with odd strides or sizes) goes to the generic kernel: a 64 x 64 x 16 LDS-tiled kernel of
+// scalar multiply-adds. Both compute a row block that straddles an expert boundary in one pass per expert, so they
+// take any padding multiple, and both check every bound.
 #include "fm_gemm_common.h"
 
 namespace fm {
@@ -42,13 +43,14 @@ constexpr int kGenTile = 64, kGenK = 16, kGenThreads = 256;
 // The work of the tile at (row0, col0) for the expert that owns its row `first_row` (relative to row0): in the
 // products whose rows are grouped by expert, a tile that straddles an expert boundary (any padding multiple is
 // allowed) is computed in one piece per expert.
-__device__ __forceinline__ TileWork resolve_tile(const GemmArgs &args, int64_t row0, int64_t col0, int first_row) {
+__device__ __forceinline__ TileWork resolve_tile(const GemmArgs &args, int64_t row0, int64_t col0, int first_row,
+                                                 int tile_rows = kGenTile) {
     TileWork work;
     work.skip = false;
     work.k_lo = 0;
     work.k_hi = args.inner;
     work.row_lo = first_row;
-    work.row_hi = kGenTile;
+    work.row_hi = tile_rows;
     work.out_offset = row0 * args.out_stride_row + col0 * args.out_stride_col;
     const bool dense = args.expert_ends == nullptr;
     if (args.mode == kInputRowSparse) {
@@ -164,6 +166,130 @@ __global__ __launch_bounds__(kGenThreads) void grouped_gemm_generic_kernel(GemmA
 }
 
 // =========================================================================================================
+// fp32 operands on the matrix cores
+// =========================================================================================================
+// 128 x 128 output tile per workgroup, 4 wavefronts (2 x 2), each 64 x 64 as 2 x 2 accumulators of
+// v_mfma_f32_32x32x2_f32 (true fp32 multiply-adds: the 1e-5 parity bound holds), K in slices of 16. Operands of any
+// strides are fetched element by element (consecutive lanes along the axis with the smaller stride) into registers
+// one slice ahead and stored to LDS as [k][row], double-buffered, one barrier per slice; several workgroups share a
+// CU. Tiles lie on a fixed 128-row grid: one that straddles an expert boundary is computed in one pass per expert,
+// like the generic kernel's, so any padding multiple works (the reference's multiple of 128 gives one pass).
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float gemm_f32x16_t;
+constexpr int kF32Tile = 128, kF32K = 16, kF32Threads = 256;
+constexpr int kF32Pitch = kF32Tile + 4;                               // floats per K-row in LDS; +4 spreads the banks
+constexpr int kF32PerThread = kF32Tile * kF32K / kF32Threads;         // operand elements per thread and slice: 8
+
+__global__ __launch_bounds__(kF32Threads) void grouped_gemm_f32_mfma_kernel(GemmArgs args) {
+    __shared__ float lds_a[2][kF32K][kF32Pitch];
+    __shared__ float lds_b[2][kF32K][kF32Pitch];
+    const int tile_n = blockIdx.x % args.tiles_n, tile_m = blockIdx.x / args.tiles_n;
+    const int64_t row0 = static_cast<int64_t>(tile_m) * kF32Tile, col0 = static_cast<int64_t>(tile_n) * kF32Tile;
+    int64_t rows_here = args.rows - row0, cols_here = args.cols - col0;
+    if (args.mode == kInputRowSparse) {
+        const int64_t left_in_expert = args.sparse_size - row0 % args.sparse_size;
+        if (left_in_expert < rows_here) rows_here = left_in_expert;
+    }
+    if (rows_here > kF32Tile) rows_here = kF32Tile;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const bool lhs_k_fastest = args.lhs_stride_inner <= args.lhs_stride_row;
+    const bool rhs_k_fastest = args.rhs_stride_inner <= args.rhs_stride_col;
+    const float *lhs_all = static_cast<const float *>(args.lhs), *rhs_all = static_cast<const float *>(args.rhs);
+
+    for (int first_row = 0; first_row < rows_here;) {
+        const TileWork work = resolve_tile(args, row0, col0, first_row, kF32Tile);
+        if (work.skip) return;  // the rest of the tile lies past the last expert
+        const int row_hi = work.row_hi < rows_here ? work.row_hi : static_cast<int>(rows_here);
+        const float *lhs = lhs_all + work.lhs_offset, *rhs = rhs_all + work.rhs_offset;
+        gemm_f32x16_t acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+        // Element e of this thread in a slice: (k, row) with the memory-contiguous axis fastest over the lanes.
+        float staged_a[kF32PerThread], staged_b[kF32PerThread];
+        auto fetch = [&](int64_t k0) {
+#pragma unroll
+            for (int e = 0; e < kF32PerThread; ++e) {
+                const int i = threadIdx.x + e * kF32Threads;
+                int k_local = lhs_k_fastest ? i % kF32K : i / kF32Tile;
+                const int r_local = lhs_k_fastest ? i / kF32K : i % kF32Tile;
+                int64_t k = k0 + k_local;
+                staged_a[e] = 0.f;
+                if (r_local >= first_row && r_local < row_hi && k >= work.k_lo && k < work.k_hi)
+                    staged_a[e] = lhs[r_local * args.lhs_stride_row + k * args.lhs_stride_inner];
+                k_local = rhs_k_fastest ? i % kF32K : i / kF32Tile;
+                const int c_local = rhs_k_fastest ? i / kF32K : i % kF32Tile;
+                k = k0 + k_local;
+                staged_b[e] = 0.f;
+                if (c_local < cols_here && k >= work.k_lo && k < work.k_hi)
+                    staged_b[e] = rhs[k * args.rhs_stride_inner + c_local * args.rhs_stride_col];
+            }
+        };
+        auto stage = [&](int buffer) {
+#pragma unroll
+            for (int e = 0; e < kF32PerThread; ++e) {
+                const int i = threadIdx.x + e * kF32Threads;
+                lds_a[buffer][lhs_k_fastest ? i % kF32K : i / kF32Tile][lhs_k_fastest ? i / kF32K : i % kF32Tile] = staged_a[e];
+                lds_b[buffer][rhs_k_fastest ? i % kF32K : i / kF32Tile][rhs_k_fastest ? i / kF32K : i % kF32Tile] = staged_b[e];
+            }
+        };
+
+        const int64_t k_begin = work.k_lo / kF32K * kF32K;
+        if (k_begin < work.k_hi) {
+            fetch(k_begin);
+            stage(0);
+        }
+        __syncthreads();
+        int buffer = 0;
+        for (int64_t k0 = k_begin; k0 < work.k_hi; k0 += kF32K, buffer ^= 1) {
+            const bool more = k0 + kF32K < work.k_hi;
+            if (more) fetch(k0 + kF32K);  // in flight during the multiplications
+#pragma unroll
+            for (int kstep = 0; kstep < kF32K / 2; ++kstep) {
+                // Lane l supplies row (or column) l % 32 at k = 2 kstep + l / 32.
+                const int k_local = 2 * kstep + (lane >> 5);
+                float a[2], b[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) a[i] = lds_a[buffer][k_local][wave_m * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) b[j] = lds_b[buffer][k_local][wave_n * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+            // The other buffer was last read a slice ago, before the previous barrier.
+            if (more) stage(buffer ^ 1);
+            __syncthreads();
+        }
+
+        // Lane l holds column l % 32 of each 32 x 32 accumulator; register v is row 8 (v / 4) + 4 (l / 32) + v % 4.
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = wave_m * 64 + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + v % 4;
+                if (row < first_row || row >= row_hi) continue;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int column = wave_n * 64 + j * 32 + (lane & 31);
+                    if (column >= cols_here) continue;
+                    store_out_dyn(args.out, args.out_dtype,
+                                  work.out_offset + row * args.out_stride_row + column * args.out_stride_col,
+                                  acc[i][j][v], args.accumulate != 0);
+                }
+            }
+        first_row = row_hi;
+        __syncthreads();  // the next pass stages into the buffers again
+    }
+}
+
+// =========================================================================================================
 // Host dispatch
 // =========================================================================================================
 static int run_gemm(const char *name, GemmArgs args, int dtype, void *workspace, size_t workspace_size, void *stream_) {
@@ -188,11 +314,19 @@ static int run_gemm(const char *name, GemmArgs args, int dtype, void *workspace,
         if (args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % kGenTile != 0)
             return fail(FM_ERR_UNSUPPORTED, "%s: row_sparse_dim=%lld must be a multiple of %d", name,
                         (long long)args.sparse_size, kGenTile);
-        args.tiles_m = static_cast<int>((args.rows + kGenTile - 1) / kGenTile);
-        args.tiles_n = static_cast<int>((args.cols + kGenTile - 1) / kGenTile);
+        // fp32 operands go to the matrix cores when the row-sparse product's blocks of out are whole tiles there too.
+        const bool f32_mfma = dtype == FM_DTYPE_F32 &&
+                              !(args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % kF32Tile != 0);
+        const int tile = f32_mfma ? kF32Tile : kGenTile;
+        args.tiles_m = static_cast<int>((args.rows + tile - 1) / tile);
+        args.tiles_n = static_cast<int>((args.cols + tile - 1) / tile);
         FM_REQUIRE(static_cast<int64_t>(args.tiles_m) * args.tiles_n < (int64_t(1) << 31), "%s: too many tiles", name);
         const int grid = args.tiles_m * args.tiles_n;
-        FM_DISPATCH_DTYPE(dtype, T, { grouped_gemm_generic_kernel<T><<<grid, kGenThreads, 0, stream>>>(args); });
+        if (f32_mfma) {
+            grouped_gemm_f32_mfma_kernel<<<grid, kF32Threads, 0, stream>>>(args);
+        } else {
+            FM_DISPATCH_DTYPE(dtype, T, { grouped_gemm_generic_kernel<T><<<grid, kGenThreads, 0, stream>>>(args); });
+        }
     }
     if (int status = check_launch(name)) return status;
     return note;
