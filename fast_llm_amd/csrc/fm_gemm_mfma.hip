@@ -450,9 +450,14 @@ __device__ __forceinline__ bool resolve_tile(const GemmArgs &args, int logical, 
 // different XCDs, so that experts with many and with few tokens (long and short tiles of the row-sparse product)
 // are spread over all of them. A permutation of every aligned block of 256 ids.
 constexpr int kRound = kXcds * kChunkTiles;  // workgroups that run at the same time: one per CU
+constexpr int kSlotRotation = 5;
 __device__ __forceinline__ int logical_of_block(int pid) {
     const int xcd = pid % kXcds, local = pid / kXcds;
-    return ((local / kChunkTiles) * kXcds + xcd) * kChunkTiles + local % kChunkTiles;
+    // Which tile of its chunk a CU takes rotates from round to round: the last row tiles of the experts, which are
+    // often half tiles and shorter, would otherwise always fall to the same CUs, and those would run further and
+    // further ahead of the CUs they share operand panels with.
+    const int round = local / kChunkTiles;
+    return (round * kXcds + xcd) * kChunkTiles + (local + round * kSlotRotation) % kChunkTiles;
 }
 
 // ---- splitting the reduction of the last tiles ---------------------------------------------------------------
