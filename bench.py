@@ -12,8 +12,8 @@ bandwidth-bound kernels, the same step with fp32 gradient buffers, the other fou
 CPU baseline (the looped torch MoE on the host cores, on a bounded token sample).
 
 `python bench.py --ceilings` prints, instead, what the device sustains: back-to-back MFMAs on zero and on random
-operands, the vendor BLAS on dense products of the same sizes, a plain streaming copy, and the rate at which the CUs
-fill LDS from L2.
+operands, the vendor BLAS on dense products of the same sizes, the library's grouped products on normal and on all-zero
+operands, a plain streaming copy, and the rate at which the CUs fill LDS from L2.
 """
 
 import argparse
@@ -277,6 +277,33 @@ def measure_ceilings(device: torch.device) -> dict:
     x_zero, weight_zero = torch.zeros_like(x), torch.zeros_like(weight)
     result["blas_dense_tflops_x_wT_zeros"] = round(gemm_flops / timed(lambda: torch.matmul(x_zero, weight_zero.t()), 10) / 1e9, 1)
     del x, weight, y, x_zero, weight_zero
+
+    # The library's three grouped products at the Mixtral shape, launched back to back on their own, on normal and on
+    # all-zero operands: on zeros the clock stays up, so the rate shows how far the kernels' structure alone would go.
+    from fast_llm_amd.functional.sparse_copy import get_sparse_map
+    from fast_llm_amd.functional.sparse_linear import (
+        input_inner_sparse_matmul,
+        input_row_sparse_matmul,
+        output_sparse_matmul,
+    )
+    from fast_llm_amd.workloads import WORKLOADS, make_inputs
+
+    workload = WORKLOADS[HEADLINE]
+    sparse_map = get_sparse_map(make_inputs(workload, weights=False).top_experts.to(device), workload.experts)
+    padded_rows, wide = sparse_map.num_rows, 2 * workload.ffn
+    grouped_flops = 2 * workload.sparse_rows_unpadded * workload.hidden * wide
+    for name, fill in (("normal_sigma_0.02", lambda t: t.normal_(0, 0.02, generator=generator)), ("zeros", lambda t: t.zero_())):
+        x = fill(torch.empty(padded_rows, workload.hidden, dtype=torch.bfloat16, device=device))
+        y = fill(torch.empty(padded_rows, wide, dtype=torch.bfloat16, device=device))
+        weight = fill(torch.empty(workload.experts * wide, workload.hidden, dtype=torch.bfloat16, device=device))
+        gradient = torch.empty_like(weight)
+        for product, function in (
+            ("output_sparse_x_wT", lambda: output_sparse_matmul(x, weight.t(), sparse_map)),
+            ("input_inner_sparse_y_w", lambda: input_inner_sparse_matmul(y, weight, sparse_map)),
+            ("input_row_sparse_yT_x", lambda: input_row_sparse_matmul(y.t(), x, sparse_map, out=gradient)),
+        ):
+            result[f"grouped_tflops_{product}_{name}"] = round(grouped_flops / timed(function, 10) / 1e9, 1)
+        del x, y, weight, gradient
 
     # Plain copies: 1 GiB read + 1 GiB written.
     size = 1 << 30
