@@ -151,8 +151,15 @@ __device__ __forceinline__ int64_t uniform_int64(int64_t value) {
 // consecutive LDS and the swizzle is applied on the global side (which chunk a lane fetches).
 // The compiler does not see these loads: whoever reads a slot counts the loads issued since (`s_waitcnt vmcnt`, loads
 // complete in order) and passes a barrier first.
-template <bool kContiguousK>
+// `kHalves` (row-contiguous only): loads 0..3 of a wavefront fill the first 32 K-rows of the slot and loads 4..7 the
+// last 32, so that either half of a slot can be refilled on its own (see the pipeline of the kernel).
+template <bool kContiguousK, bool kHalves = false>
 struct TileLoader {
+    static_assert(!(kContiguousK && kHalves), "only a row-contiguous slice splits into halves along K");
+    // The 1 KiB block of an operand slot that load j of wavefront `wave` fills.
+    static __device__ __forceinline__ int block_of(int wave, int j) {
+        return kHalves ? (j >> 2) * (2 * kLoadsPerOperand) + wave * (kLoadsPerOperand / 2) + (j & 3) : wave * kLoadsPerOperand + j;
+    }
     const char *fetch_base;  // wave-uniform: first row of the tile, first k of the slice being fetched
     uint32_t offset[2];      // per lane, bytes from `fetch_base`, of loads 0 and 1 (fits 32 bits: checked on the host)
     uint32_t pair_stride;    // wave-uniform: bytes from load j to load j + 2 (the swizzles repeat with period 2)
@@ -161,7 +168,7 @@ struct TileLoader {
     int slices_left;         // slices after the one being fetched
     uint32_t last_records;   // row-contiguous: `num_records` of the last slice (its K-rows past the reduction range
                              // bring zeros)
-    int lds_offset;          // wave-uniform: of this wavefront's first 1 KiB block within an operand slot
+    int wave_index;          // wave-uniform
 
     // `stride`: bytes between rows (K-contiguous) or between K-rows (row-contiguous). Rows >= valid_rows are never
     // stored; a K-contiguous operand gets zeros for them (they lie past the range of the buffer descriptor), a
@@ -176,10 +183,10 @@ struct TileLoader {
         static_assert(kLoadsPerOperand % 2 == 0, "loads come in (even, odd) pairs");
         fetch_base = tile_base;
         slices_left = num_slices - 1;
-        lds_offset = wave * kLoadsPerOperand * 1024;
+        wave_index = wave;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const int slot = (wave * kLoadsPerOperand + j) * 64 + lane;
+            const int slot = block_of(wave, j) * 64 + lane;
             if constexpr (kContiguousK) {
                 const int row = slot / kChunksPerRow;
                 const int chunk = (slot % kChunksPerRow) ^ k_major_swizzle(row);
@@ -222,8 +229,11 @@ struct TileLoader {
         const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<char *>(uniform_pointer(fetch_base)), 0,
             static_cast<int>(__builtin_amdgcn_readfirstlane(num_records)), kBufferResourceFlags);
-        const uint32_t lane_offset = offset[j & 1] + static_cast<uint32_t>(j >> 1) * pair_stride;
-        const int block_address = __builtin_amdgcn_readfirstlane(slot_address + lds_offset + j * 1024);
+        // Two loads further on the blocks are two further on (`pair_stride`); with halves, four loads further on they
+        // are 16 further on: 32 K-rows, eight times the four K-rows of `pair_stride`.
+        const uint32_t lane_offset =
+            offset[j & 1] + static_cast<uint32_t>(kHalves ? ((j >> 1) & 1) + 8 * (j >> 2) : j >> 1) * pair_stride;
+        const int block_address = __builtin_amdgcn_readfirstlane(slot_address + block_of(wave_index, j) * 1024);
         // M0 is not handed out by the register allocator and nothing else in this file uses it.
         asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      :
@@ -626,6 +636,9 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
     constexpr int kRowBytes = kWaveCols * sizeof(StageT) + kEpiloguePadBytes;
     const int wave_n = wave % kWavesN;
     FM_LDS(char) *staging = lds + wave * (32 * kRowBytes);
+    // (Two-byte values: a lane writes 8 bytes and the rows are 272 bytes apart, so rows r and r + 16 meet in the same
+    // banks: two-way conflicts on these writes. Swapping the halves of every 16-byte chunk in half of the rows removes
+    // them, measured with the bank-conflict counter, and the kernel is no faster for it: not done.)
     FM_LDS(char) *write_base = staging + (lane & 31) * kRowBytes + (lane >> 5) * 4 * sizeof(StageT);
     const int read_row = lane / kLanesPerRow, read_column = (lane % kLanesPerRow) * kChunk;
     FM_LDS(char) *read_base = staging + read_row * kRowBytes + read_column * sizeof(StageT);
@@ -913,6 +926,19 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     // previous tile is written out. Ids map to tiles in increasing order, so the first id without a tile ends the walk.
     // Everything about a tile is the same in every lane and is said to be, so that it lives in scalar registers.
     constexpr bool kSlicesFromRangeStart = kMasked && !kLhsContiguousK && !kRhsContiguousK;
+    // The halves of a row-contiguous rhs slot are refilled separately (not where a slice may need masking in LDS, which
+    // works on whole slices that have landed).
+    // When the loads of the rhs slices are issued (see the pipeline below). Measured per product on the 12 to 64
+    // slice reductions of the fine-grained and wide workloads: -1..-5 % for the two unmasked products; the
+    // weight-gradient product gains nothing from either of the other two schedules.
+    constexpr int kScheduleSplit = 0, kScheduleLate = 1, kScheduleHalves = 2;
+    constexpr int kSchedule = kMasked ? kScheduleSplit : (kRhsContiguousK ? kScheduleLate : kScheduleHalves);
+    constexpr bool kRhsHalves = kSchedule == kScheduleHalves;
+    // Loads that may still be on their way at the barrier before the last K-step and at the one after K-step 0.
+    constexpr int kBarrierNewest = kSchedule == kScheduleSplit ? 6 : (kSchedule == kScheduleLate ? 8 : 16);
+    constexpr int kMidBarrierNewest = 18;
+    typedef TileLoader<kLhsContiguousK> LhsLoader;
+    typedef TileLoader<kRhsContiguousK, kRhsHalves> RhsLoader;
     struct Tile {
         TileRecord work;
         int piece_slot;   // >= 0: a piece of a split reduction, stored to that workspace slot
@@ -950,8 +976,8 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     Tile tile;
     if (id >= args.num_ids || !find_tile(id, tile)) return;
 
-    TileLoader<kLhsContiguousK> load_lhs;
-    TileLoader<kRhsContiguousK> load_rhs;
+    LhsLoader load_lhs;
+    RhsLoader load_rhs;
 
     f32x16_t acc[kTilesM][kTilesN];
     auto clear_accumulators = [&]() {
@@ -965,16 +991,23 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
 
     // ---- the software pipeline --------------------------------------------------------------------------
     // A slot that is being filled cannot be read, and LDS (160 KiB) has room for five operand slices of 32 KiB: three
-    // lhs slots and two rhs slots. During iteration t (multiplying slice t; rhs slot t % 2, lhs slot t % 3):
-    //   K-step 0     : rhs chunks 4..7 of slice t + 1 are loaded (into the slot slice t - 1 left);
-    //   K-steps 0..2 : lhs chunks 2..7 of slice t + 2 are loaded, two per K-step, into lhs slot (t + 2) % 3;
-    //   barrier      : every wavefront has waited for all its loads but the 6 newest (the lhs loads of this
-    //                  iteration), so slice t + 1 is complete and visible; nobody reads the slots of slice t any more
-    //                  except through fragments already in registers (those of K-step 3 were read during K-step 2);
-    //   K-step 3     : rhs chunks 0..3 of slice t + 2 and lhs chunks 0, 1 of slice t + 3 are loaded into the slots
-    //                  slice t just left; the fragments of K-step 0 of slice t + 1 are read.
-    // So an lhs load has a slice or more to land and an rhs load half a slice or more (measured on the predecessor of
-    // this pipeline: capping the loads in flight at half a slice per wavefront costs nothing, a quarter costs 6 %).
+    // lhs slots and two rhs slots. Iteration t multiplies slice t (rhs slot t % 2, lhs slot t % 3) in four K-steps. The
+    // barrier before K-step 3 makes slice t + 1 visible and ends the reads of slice t's slots (the fragments of K-step 3
+    // are in registers by then). The loads of a wavefront complete in order, and before a barrier a wavefront waits
+    // until all but its N newest loads have landed; N counts the loads issued since the newest one that the reads
+    // after the barrier need. Every K-step issues two lhs loads: chunks 2..7 of slice t + 2 in K-steps 0..2, chunks
+    // 0, 1 of slice t + 3 in K-step 3 (into the slot slice t just left). The rhs loads follow one of three schedules:
+    //   split  : chunks 4..7 of slice t + 1 in K-step 0, chunks 0..3 of slice t + 2 in K-step 3; N = 6. An rhs load
+    //            has half a slice of MFMAs or more to land.
+    //   late   : all 8 chunks of slice t + 2 in K-step 3, right after the barrier that frees their slot, and the lhs
+    //            loads of slice t + 2 in K-steps 0..2 (three, three, two); N = 8, three quarters of a slice for an rhs load.
+    //   halves : a row-contiguous rhs slot is refilled in halves (K-rows 0..31, 32..63). A second barrier, after K-step
+    //            0, makes the second half of slice t visible and ends the reads of its first half (N = 18); every
+    //            K-step then issues two rhs loads: chunks 6, 7 of slice t + 1 in K-step 0, chunks 0..5 of slice t + 2
+    //            in K-steps 1..3 (0..3 are its first half), and N = 16 at the barrier before K-step 3. Every load has a
+    //            full slice of MFMAs to land, and the loads are spread evenly over the K-steps.
+    // A K-contiguous rhs slice does not split along K (a row's 128 bytes are one cache line). Which schedule an instance
+    // uses was measured (`kSchedule`).
     // Fragments are double-buffered over K-steps, across slices as well. There is no branch around a transfer: loads
     // past the last slice bring zeros.
     u32x4_t frag_a[2][kTilesM], frag_b[2][kTilesN];
@@ -1009,54 +1042,79 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     // with a scheduling barrier after every slot:
     //   slots 0..3     rhs fragments 0..3 of the next K-step (other fragment buffer)
     //   slots 4..7     lhs fragments 0..3 of the next K-step
-    //   slots 8..11    in K-steps 0 and 3: four rhs loads
-    //   slots 12, 13   two lhs loads
+    //   slots 8..11    rhs loads (schedule "late": slots 8..15 of K-step 3)
+    //   slots 12..14   lhs loads
     // A half tile has 8 slots per K-step (2 x 4 accumulators): rhs fragments in slots 0..3, the two lhs fragments in
-    // slots 4, 5, the rhs loads in slots 2..5 as well and the lhs loads in slots 6, 7.
+    // slots 4, 5, the rhs loads in slots 2..5 as well ("late": two per slot) and the lhs loads from slot 5 on.
     static_assert(kTilesM == 4 && kTilesN == 4 && kLoadsPerOperand == 8, "the slot table below is written for this shape");
     auto iteration = [&](int t, auto slot_constant, auto half_constant) {
         constexpr int kSlot = decltype(slot_constant)::value, kNextSlot = 1 - kSlot;  // rhs, of slices t, t + 1
         constexpr bool kHalf = decltype(half_constant)::value;
         constexpr int kRowBlocks = kHalf ? kTilesM / 2 : kTilesM;
+        constexpr int kSlots = kRowBlocks * kTilesN;
+        constexpr int kRhsLoadSlot = kHalf ? 2 : 8;  // first slot of a K-step that issues rhs loads
+        constexpr int kLhsLoadSlot = kHalf ? 5 : 12;  // first slot of a K-step that issues lhs loads
 #pragma unroll
         for (int kstep = 0; kstep < kSteps; ++kstep) {
             const bool last = kstep + 1 == kSteps;
             const int next_slot = last ? kNextSlot : kSlot, next_kstep = (kstep + 1) % kSteps;
             const int buffer = kstep & 1;
-            // The lhs chunks loaded during this K-step: 2..7 of slice t + 2, then 0, 1 of slice t + 3.
-            const int lhs_chunk = 2 * next_kstep, lhs_target = last ? lhs_now : lhs_after;
-            if (last) {
-                load_lhs.advance();
-                load_rhs.advance();
+            // What this K-step loads (see the table above): `lhs_count` lhs chunks from `lhs_chunk` on, `rhs_count` rhs
+            // chunks from `rhs_chunk` on into rhs slot `rhs_slot`.
+            int lhs_chunk = 0, lhs_count = 0, lhs_target = lhs_after, rhs_chunk = 0, rhs_count = 0, rhs_slot = kSlot;
+            if constexpr (kSchedule == kScheduleSplit) {
+                lhs_chunk = 2 * next_kstep, lhs_count = 2;
+                if (last) {
+                    load_lhs.advance();
+                    load_rhs.advance();
+                    lhs_target = lhs_now;
+                    rhs_count = 4;
+                } else if (kstep == 0) {
+                    rhs_chunk = 4, rhs_count = 4, rhs_slot = kNextSlot;
+                }
+            } else if constexpr (kSchedule == kScheduleLate) {
+                lhs_chunk = 3 * kstep, lhs_count = kstep < 2 ? 3 : (last ? 0 : 2);
+                if (kstep == 0) load_lhs.advance();
+                if (last) {
+                    load_rhs.advance();
+                    rhs_count = 8;
+                }
+            } else {
+                lhs_chunk = 2 * next_kstep, lhs_count = 2;
+                rhs_chunk = kstep == 0 ? 6 : 2 * (kstep - 1), rhs_count = 2;  // 6, 7 of slice t + 1, then 0..5 of slice t + 2
+                if (kstep == 0) rhs_slot = kNextSlot;
+                if (kstep == 1) load_rhs.advance();
+                if (last) {
+                    load_lhs.advance();
+                    lhs_target = lhs_now;
+                }
             }
 #pragma unroll
-            for (int m = 0; m < kRowBlocks * kTilesN; ++m) {
+            for (int m = 0; m < kSlots; ++m) {
                 // Boustrophedon order: consecutive MFMAs always share one operand (fewer operand-bus toggles).
                 const int i = m / kTilesN, j = (i & 1) ? kTilesN - 1 - m % kTilesN : m % kTilesN;
                 acc[i][j] = Mfma<T>::run(frag_b[buffer][j], frag_a[buffer][i], acc[i][j]);  // transposed, see store_tile
-                if constexpr (kHalf) {
-                    if (m < 4) read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
-                    else if (m < 6) read_lhs_fragment(last, next_kstep, buffer ^ 1, m - 4);
-                    // All rhs loads of a K-step before its lhs loads: the wait before the barrier counts on it.
-                    if (m >= 2 && m < 6) {
-                        if (kstep == 0) load_rhs.load(kNextSlot * kOperandBytes, 4 + m - 2);
-                        else if (last) load_rhs.load(kSlot * kOperandBytes, m - 2);
+                if (m < kTilesN) read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
+                else if (m < kTilesN + kRowBlocks) read_lhs_fragment(last, next_kstep, buffer ^ 1, m - kTilesN);
+                // All rhs loads of a K-step before its lhs loads: the waits before the barriers count on it.
+                if (kHalf && rhs_count == 8) {  // two per slot
+                    if (m >= kRhsLoadSlot && m < kRhsLoadSlot + 4) {
+                        load_rhs.load(rhs_slot * kOperandBytes, 2 * (m - kRhsLoadSlot));
+                        load_rhs.load(rhs_slot * kOperandBytes, 2 * (m - kRhsLoadSlot) + 1);
                     }
-                    if (m >= 6) load_lhs.load(lhs_target, lhs_chunk + m - 6);
-                } else if (m < 4) {
-                    read_rhs_fragment(next_slot, next_kstep, buffer ^ 1, m);
-                } else if (m < 8) {
-                    read_lhs_fragment(last, next_kstep, buffer ^ 1, m - 4);
-                } else if (m < 12) {
-                    if (kstep == 0) load_rhs.load(kNextSlot * kOperandBytes, 4 + m - 8);
-                    else if (last) load_rhs.load(kSlot * kOperandBytes, m - 8);
-                } else if (m < 14) {
-                    load_lhs.load(lhs_target, lhs_chunk + m - 12);
+                } else if (m >= kRhsLoadSlot && m < kRhsLoadSlot + rhs_count) {
+                    load_rhs.load(rhs_slot * kOperandBytes, rhs_chunk + m - kRhsLoadSlot);
                 }
+                if (m >= kLhsLoadSlot && m < kLhsLoadSlot + lhs_count)
+                    load_lhs.load(lhs_target, lhs_chunk + m - kLhsLoadSlot);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if (kRhsHalves && kstep == 0) {
+                wait_for_loads<kMidBarrierNewest>();
+                __syncthreads();
+            }
             if (kstep == kSteps - 2) {
-                wait_for_loads<6>();
+                wait_for_loads<kBarrierNewest>();
                 __syncthreads();
                 mask_slice(t + 1, lhs_next, kNextSlot);
             }
@@ -1073,12 +1131,11 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         }
     };
     // The loads that start a tile come in two parts: slice 0 of both operands (16 loads per wavefront), which are issued
-    // while the previous tile is still being written out, and the 14 loads that follow (lhs slice 1, rhs chunks 0..3
-    // of slice 1, lhs chunks 0, 1 of slice 2). Nothing that `first_loads` computes per lane outlives it: the loaders
-    // and fragment addresses of the tile are set up (again) by `setup_tile`, after the previous tile's epilogue, so
-    // that they do not occupy registers during it.
-    auto setup_loaders = [&](const Tile &next, TileLoader<kLhsContiguousK> &lhs_loader,
-                             TileLoader<kRhsContiguousK> &rhs_loader, int lane) {
+    // while the previous tile is still being written out, and those that follow (`continue_tile`: slice 1 of both
+    // operands and, with rhs halves, lhs chunks 0, 1 of slice 2), in the order the main loop would have issued them.
+    // Nothing that `first_loads` computes per lane outlives it: the loaders and fragment addresses of the tile are set
+    // up (again) by `setup_tile`, after the previous tile's epilogue, so that they do not occupy registers during it.
+    auto setup_loaders = [&](const Tile &next, LhsLoader &lhs_loader, RhsLoader &rhs_loader, int lane) {
         const TileRecord &work = next.work;
         const char *lhs = static_cast<const char *>(args.lhs) +
                           (work.lhs_offset + next.k_first * args.lhs_stride_inner) * static_cast<int64_t>(sizeof(T));
@@ -1095,8 +1152,8 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     constexpr int kFirstLhsSlot = kLhsBase + (kLhsStages - 1) * kOperandBytes;
     auto first_loads = [&](const Tile &next) {
         if (next.num_slices <= 0) return;
-        TileLoader<kLhsContiguousK> lhs_loader;
-        TileLoader<kRhsContiguousK> rhs_loader;
+        LhsLoader lhs_loader;
+        RhsLoader rhs_loader;
         setup_loaders(next, lhs_loader, rhs_loader, opaque(lane));
 #pragma unroll
         for (int j = 0; j < kLoadsPerOperand; ++j) lhs_loader.load(kFirstLhsSlot, j);
@@ -1118,17 +1175,23 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             rhs_frag[q] = fragment_base<kRhsContiguousK>(wave_n * kWaveCols, q, lane);
         }
     };
+    // rhs chunks of slice 1 and lhs chunks of slice 2 that the prologue issues (the main loop issues the rest).
+    constexpr int kPrologueRhs = kSchedule == kScheduleSplit ? 4 : (kSchedule == kScheduleHalves ? 6 : 8);
+    constexpr int kPrologueLhs = kSchedule == kScheduleLate ? 0 : 2;
     auto continue_tile = [&]() {
         load_lhs.advance();
         load_rhs.advance();
 #pragma unroll
         for (int j = 0; j < kLoadsPerOperand; ++j) load_lhs.load(lhs_next, j);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) load_rhs.load(kOperandBytes, j);
-        load_lhs.advance();
+        for (int j = 0; j < kPrologueRhs; ++j) load_rhs.load(kOperandBytes, j);
+        if constexpr (kPrologueLhs > 0) {
+            load_lhs.advance();
 #pragma unroll
-        for (int j = 0; j < 2; ++j) load_lhs.load(lhs_after, j);
+            for (int j = 0; j < kPrologueLhs; ++j) load_lhs.load(lhs_after, j);
+        }
     };
+    constexpr int kLoadsAfterSlice0 = kLoadsPerOperand + kPrologueRhs + kPrologueLhs;
 
     first_loads(tile);
     while (true) {
@@ -1138,7 +1201,7 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             // Prologue: slice 0, lhs slice 1 and the first pieces of the slices after them on their way; slice 0 landed.
             continue_tile();
             clear_accumulators();  // 256 register writes, while the first loads are on their way
-            wait_for_loads<14>();  // 30 loads since the tile began, the first 16 of them slice 0
+            wait_for_loads<kLoadsAfterSlice0>();  // slice 0 was loaded first
             __syncthreads();
             mask_slice(0, lhs_now, 0);
 #pragma unroll
