@@ -713,6 +713,11 @@ __device__ __forceinline__ void store_tile(Source &&source, FM_LDS(char) * lds, 
         else store_rows(std::false_type{});
         asm volatile("" ::: "memory");
     }
+    // vmcnt(0). The compiler cannot tell that every load above has been waited for (loads and uses sit in separate
+    // conditionals) and would otherwise wait for all memory operations at the top of the caller's tile loop, in
+    // launches that do not accumulate as well: there that wait held a tile's first transfers back until the previous
+    // tile's stores had been acknowledged.
+    if constexpr (kAccumulate) __builtin_amdgcn_s_waitcnt(0x0F70);
 }
 
 // ---- fused epilogues of the gated MLP ---------------------------------------------------------------------
