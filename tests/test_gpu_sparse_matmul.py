@@ -304,6 +304,47 @@ def test_mfma_kernel_on_ragged_experts(experts, dense_dim, sparse_dim, dtype, de
         assert max_rel_err(out.cpu(), 2 * expected.float()) <= tolerance
 
 
+# The matrix-core kernel counts by hand which of its transfers have landed when a K-step reads them, with one count
+# per load schedule (K-contiguous rhs, row-contiguous rhs, weight gradient) and tile kind (whole, half: an expert's last
+# row tile with at most 128 valid rows). Every number of 64-wide reduction slices from 1 to 10 through all of them:
+# experts of 256 + 128 rows (a whole and a half tile), of 128 rows (a half tile) and of 512 rows; the walk of a
+# workgroup over several tiles comes with the 40 column tiles of the second size.
+@pytest.mark.parametrize("slices", range(1, 11))
+@pytest.mark.parametrize("other", [256, 40 * 256])
+def test_every_slice_count_through_the_pipeline(slices, other, device):
+    if other > 256 and slices not in (1, 2, 3, 6, 9):
+        pytest.skip("the long walk is run for a few slice counts only")
+    dtype = torch.bfloat16
+    inner = 64 * slices
+    case = {"expert_ends": [384, 512, 1024], "tokens_per_expert": [300, 77, 512], "phantom_rows": 128}
+    oracle_map = fixture_sparse_map(case)
+    oracle_map.num_rows = case["expert_ends"][-1] + case["phantom_rows"]
+    sparse_map = to_device_map(oracle_map, device, torch.int32)
+    used = _used_rows(oracle_map)
+    experts = len(case["expert_ends"])
+    generator = torch.Generator().manual_seed(slices)
+    x = _normal(oracle_map.num_rows, inner, dtype, generator)
+    x[~oracle_map.real_row_mask()] = 0
+    x_gpu = x.to(device)
+
+    weight = _normal(experts * other, inner, dtype, generator)  # K-contiguous rhs
+    out = output_sparse_matmul(x_gpu, weight.to(device).t(), sparse_map)
+    expected = moe_oracle.output_sparse_matmul(x, weight.t(), oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= _MAX_REL[dtype]
+
+    weight = _normal(experts * inner, other, dtype, generator)  # row-contiguous rhs
+    out = input_inner_sparse_matmul(x_gpu, weight.to(device), sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(x, weight, oracle_map)
+    assert max_rel_err(out[:used].cpu(), expected[:used]) <= _MAX_REL[dtype]
+
+    if other == 256:  # the weight gradient: its reduction runs over the rows, 1 .. 8 slices here; 128 x 256 outputs
+        y = _normal(oracle_map.num_rows, other, dtype, generator)
+        narrow = _normal(oracle_map.num_rows, 128, dtype, generator)
+        out = input_row_sparse_matmul(narrow.to(device).t(), y.to(device), sparse_map)
+        expected = moe_oracle.input_row_sparse_matmul(narrow.t(), y, oracle_map)
+        assert max_rel_err(out.cpu(), expected) <= _MAX_REL[dtype]
+
+
 # Few tiles and a long reduction: the tiles of the last round of workgroups are cut along the reduction axis and their
 # pieces added by a second kernel. (experts, reduction size, other size): 4 pieces of 18 slices with a shorter, odd last
 # one; whole tiles followed by more than 256 pieces; 2 pieces.
