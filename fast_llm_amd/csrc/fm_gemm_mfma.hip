@@ -931,11 +931,10 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     // previous tile is written out. Ids map to tiles in increasing order, so the first id without a tile ends the walk.
     // Everything about a tile is the same in every lane and is said to be, so that it lives in scalar registers.
     constexpr bool kSlicesFromRangeStart = kMasked && !kLhsContiguousK && !kRhsContiguousK;
-    // The halves of a row-contiguous rhs slot are refilled separately (not where a slice may need masking in LDS, which
-    // works on whole slices that have landed).
     // When the loads of the rhs slices are issued (see the pipeline below). Measured per product on the 12 to 64
     // slice reductions of the fine-grained and wide workloads: -1..-5 % for the two unmasked products; the
-    // weight-gradient product gains nothing from either of the other two schedules.
+    // weight-gradient product gains nothing from either of the other two schedules, and a product that masks slices in
+    // LDS works on whole slices that have landed.
     constexpr int kScheduleSplit = 0, kScheduleLate = 1, kScheduleHalves = 2;
     constexpr int kSchedule = kMasked ? kScheduleSplit : (kRhsContiguousK ? kScheduleLate : kScheduleHalves);
     constexpr bool kRhsHalves = kSchedule == kScheduleHalves;
@@ -1000,8 +999,9 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     // barrier before K-step 3 makes slice t + 1 visible and ends the reads of slice t's slots (the fragments of K-step 3
     // are in registers by then). The loads of a wavefront complete in order, and before a barrier a wavefront waits
     // until all but its N newest loads have landed; N counts the loads issued since the newest one that the reads
-    // after the barrier need. Every K-step issues two lhs loads: chunks 2..7 of slice t + 2 in K-steps 0..2, chunks
-    // 0, 1 of slice t + 3 in K-step 3 (into the slot slice t just left). The rhs loads follow one of three schedules:
+    // after the barrier need. Except under "late", every K-step issues two lhs loads: chunks 2..7 of slice t + 2 in
+    // K-steps 0..2, chunks 0, 1 of slice t + 3 in K-step 3 (into the slot slice t just left). The rhs loads follow one
+    // of three schedules:
     //   split  : chunks 4..7 of slice t + 1 in K-step 0, chunks 0..3 of slice t + 2 in K-step 3; N = 6. An rhs load
     //            has half a slice of MFMAs or more to land.
     //   late   : all 8 chunks of slice t + 2 in K-step 3, right after the barrier that frees their slot, and the lhs
