@@ -8,15 +8,22 @@ configuration (8192 tokens, hidden 4096, ffn 14336, 8 experts, top-2, bf16 with 
 
 Prints one JSON line: whole-step tokens/s, the roofline of the grouped-GEMM kernel (six launches per step, algorithmic
 FLOPs 18*M*H*F over their summed device time from HIP events on the launch stream), per-kernel figures for the
-bandwidth-bound kernels, the same step with fp32 gradient buffers, the other four configurations (`configs`), and a
-CPU baseline (the looped torch MoE on the host cores, on a bounded token sample).
+bandwidth-bound kernels (mean, median and minimum over the timed steps), `box` (what this very device sustains in the
+same run: a register-only MFMA loop on random operands and the shader clock it holds), `isolated` (every kernel of the
+step launched on its own with the caches flushed in between: median and minimum of 20 launches), the same step with
+fp32 gradient buffers and with full recomputation, the other four configurations (`configs`), and a CPU baseline (the
+looped torch MoE on the host cores over the whole batch).
 
 `python bench.py --ceilings` prints, instead, what the device sustains: back-to-back MFMAs on zero and on random
 operands, the vendor BLAS on dense products of the same sizes, the library's grouped products on normal and on all-zero
 operands, a plain streaming copy, and the rate at which the CUs fill LDS from L2.
+
+The probes behind `box` and `--ceilings` are not part of the kernel library: they are `bench_probes.hip` beside this
+file, built into `libbench_probes.so` by `build_probes()` (which `__graft_entry__.build()` calls).
 """
 
 import argparse
+import ctypes
 import json
 import os
 import pathlib
@@ -29,8 +36,12 @@ import torch
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak, TFLOP/s
 PEAK_FP32_TFLOPS = 157.3  # MI355X fp32 (matrix) peak, TFLOP/s
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E peak, GB/s
-PROFILES = pathlib.Path(__file__).resolve().parent / "profiles"
+ROOT = pathlib.Path(__file__).resolve().parent
+PROFILES = ROOT / "profiles"
+PROBE_SOURCE, PROBE_LIBRARY = ROOT / "bench_probes.hip", ROOT / "libbench_probes.so"
+FLUSH_BYTES = 512 << 20  # written between isolated launches: twice the 256 MiB Infinity Cache
 HEADLINE = "mixtral"
+_ISOLATED_KEYS = ("ms_median", "ms_min", "tflops", "frac_of_mfma_peak", "gbs", "frac_of_hbm_peak")
 OTHER_WORKLOADS = ("tiny", "fine_grained", "wide", "imbalanced")
 
 
@@ -46,6 +57,71 @@ def measured_traffic(workload_name: str) -> tuple[int | None, str | None]:
     return summary["traffic_bytes_per_launch"], summary["source"]
 
 
+def build_probes(verbose: bool = True) -> pathlib.Path:
+    """Compile `bench_probes.hip` for gfx950 into `libbench_probes.so` (no GPU needed)."""
+    if str(ROOT) not in sys.path:
+        sys.path.insert(0, str(ROOT))
+    from fast_llm_amd.build import build_shared
+
+    return build_shared([PROBE_SOURCE], PROBE_LIBRARY, verbose)
+
+
+_probes: ctypes.CDLL | None = None
+
+
+def probes() -> ctypes.CDLL:
+    """The probe library, built first if it is not there."""
+    global _probes
+    if _probes is None:
+        if not PROBE_LIBRARY.is_file():
+            build_probes()
+        library = ctypes.CDLL(str(PROBE_LIBRARY))
+        i64, ptr = ctypes.c_int64, ctypes.c_void_p
+        library.probe_mfma.argtypes = [ptr, ptr, i64, i64, ctypes.c_int, ctypes.c_float, ptr]
+        library.probe_mfma_flops.argtypes, library.probe_mfma_flops.restype = [i64, i64], i64
+        library.probe_copy.argtypes = [ptr, ptr, i64, i64, ptr]
+        library.probe_l2.argtypes = [ptr, i64, i64, i64, i64, i64, ptr, ptr]
+        _probes = library
+    return _probes
+
+
+def probe_ok(status: int) -> None:
+    if status != 0:
+        raise RuntimeError(f"probe launch failed with status {status}")
+
+
+def box_probe(device: torch.device, launches: int = 3) -> dict:
+    """What this device sustains right now: a register-only loop of the grouped products' MFMA instruction on
+    normal(0, 0.02) bf16 operands on every CU (about 40 ms per launch), and the shader clock it holds meanwhile. The
+    chip is power-limited, boxes differ by a few per cent, and this is the ceiling of the one the figures come from."""
+    library = probes()
+    stream = torch.cuda.current_stream(device)
+    compute_units = torch.cuda.get_device_properties(device).multi_processor_count
+    iterations = 40000
+    sink = torch.empty(compute_units * 256, dtype=torch.float32, device=device)
+    cycles = torch.zeros(compute_units, dtype=torch.int64, device=device)
+
+    def launch() -> None:
+        probe_ok(library.probe_mfma(sink.data_ptr(), cycles.data_ptr(), compute_units, iterations, 1, 0.02, stream.cuda_stream))
+
+    launch()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for _ in range(launches):
+        launch()
+    end.record(stream)
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / launches
+    tflops = library.probe_mfma_flops(compute_units, iterations) / ms / 1e9
+    return {
+        "mfma_loop_tflops_random": round(tflops, 1),
+        "mfma_loop_frac_of_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "shader_clock_mhz": round(cycles.double().mean().item() / ms / 1e3),
+        "what": f"{launches} launches of {iterations} x 32 back-to-back v_mfma_f32_32x32x16_bf16 per wavefront, 4 "
+        f"wavefronts on each of {compute_units} CUs, normal(0, 0.02) operands in registers, right after the timed steps",
+    }
+
+
 def parse_args() -> argparse.Namespace:
     parser = argparse.ArgumentParser(description=__doc__)
     parser.add_argument("--gpus", type=int, default=1)
@@ -54,8 +130,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--workload", default=HEADLINE, help="tiny | mixtral | fine_grained | wide | imbalanced")
     parser.add_argument("--recompute", default="none", help="none | activation | activation_and_input | full")
     parser.add_argument(
-        "--cpu-tokens", type=int, default=4096, help="tokens in the CPU baseline sample of the headline (0: skip)"
-    )
+        "--cpu-tokens", type=int, default=1 << 30,
+        help="tokens in the CPU baseline sample of the headline, at most the whole batch (the default; 0: skip)",
+    )  # fmt: skip
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument(
         "--grad-dtype",
@@ -148,43 +225,22 @@ def time_workload(workload, args, steps: int, warmup: int, grad_dtype_name: str,
         torch.cuda.synchronize()
         seconds = time.perf_counter() - start
     ms_per_step = seconds / steps * 1e3
-
-    # Per-kernel device time, averaged over the timed steps.
     all_durations = timer.durations_ms()
-    durations = {label: sum(values) / len(values) for label, values in all_durations.items()}
     calls_per_step = {label: len(values) / steps for label, values in all_durations.items()}
-    rows, hidden, ffn = workload.sparse_rows_unpadded, workload.hidden, workload.ffn
-    itemsize = workload.dtype.itemsize
+    kernels = {
+        label: kernel_figures(label, values, workload, recompute_level) | {"calls_per_step": calls_per_step[label]}
+        for label, values in sorted(all_durations.items())
+    }
+    # Whole-step GEMM rate: algorithmic FLOPs of a step over the summed mean launch times.
     peak_tflops = PEAK_FP32_TFLOPS if workload.dtype == torch.float32 else PEAK_BF16_TFLOPS
-    gemm_ms = sum(durations[label] * calls_per_step[label] for label in durations if "matmul" in label)
-    gemm_launches = sum(calls_per_step[label] for label in durations if "matmul" in label)
+    gemm_ms = sum(kernels[label]["ms"] * calls_per_step[label] for label in kernels if "matmul" in label)
+    gemm_launches = sum(calls_per_step[label] for label in kernels if "matmul" in label)
     gemm_flops = workload.gemm_flops * (4 / 3 if recompute_level.recompute_layer_1 else 1)
     gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12
-    index_size = 2 if rows + workload.experts * 128 < 32768 else 4
-    copy_bytes = workload.copy_bytes + rows * (index_size + 4)  # rows + indices + fp32 scores
-    kernels = {}
-    for label, ms in sorted(durations.items()):
-        entry = {"ms": round(ms, 4), "calls_per_step": calls_per_step[label]}
-        if "matmul" in label:
-            m, n, k = (int(v) for v in label[label.index("[") + 1 : -1].split("x"))
-            # Dimensions are padded/static; algorithmic FLOPs use the unpadded row count.
-            per_launch = 2 * rows * (n if "row_sparse" not in label else m) * (k if "row_sparse" not in label else n)
-            entry["tflops"] = round(per_launch / (ms * 1e-3) / 1e12, 1)
-            entry["frac_of_mfma_peak"] = round(entry["tflops"] / peak_tflops, 4)
-        elif label in ("fm_copy_dense_to_sparse", "fm_copy_sparse_to_dense"):
-            entry["gbs"] = round(copy_bytes / (ms * 1e-3) / 1e9, 1)
-            entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
-        elif label == "fm_copy_sparse_to_dense_backward":
-            fused_bytes = (1 + 2 * workload.experts_per_token) * workload.tokens * hidden * itemsize
-            entry["gbs"] = round(fused_bytes / (ms * 1e-3) / 1e9, 1)
-            entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
-        elif label.startswith("fm_mlp_activation"):
-            factor = 3 if label.endswith("forward") else (6 if recompute_level.recompute_activation else 5)
-            entry["gbs"] = round(factor * rows * ffn * itemsize / (ms * 1e-3) / 1e9, 1)
-            entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
-        kernels[label] = entry
     return {
         "inputs": inputs,
+        "step": step,
+        "state": (x, scores, weight_1, weight_2),
         "ms_per_step": ms_per_step,
         "tokens_per_s": workload.tokens * steps / seconds,
         "gemm_ms": gemm_ms,
@@ -194,6 +250,134 @@ def time_workload(workload, args, steps: int, warmup: int, grad_dtype_name: str,
         "gemm_peak_tflops": peak_tflops,
         "kernels": kernels,
     }
+
+
+def kernel_figures(label: str, durations_ms: list[float], workload, recompute_level) -> dict:
+    """Mean, median and minimum device time of the launches of one kernel-library call, and the rate its algorithmic
+    work (unpadded rows) gives at the mean, as a fraction of the matrix peak or of the HBM peak."""
+    ms = sum(durations_ms) / len(durations_ms)
+    entry = {
+        "ms": round(ms, 4),
+        "ms_median": round(statistics.median(durations_ms), 4),
+        "ms_min": round(min(durations_ms), 4),
+    }
+    rows, hidden, ffn = workload.sparse_rows_unpadded, workload.hidden, workload.ffn
+    itemsize = workload.dtype.itemsize
+    peak_tflops = PEAK_FP32_TFLOPS if workload.dtype == torch.float32 else PEAK_BF16_TFLOPS
+    index_size = 2 if rows + workload.experts * 128 < 32768 else 4
+    work_bytes = None
+    if "matmul" in label:
+        m, n, k = (int(v) for v in label[label.index("[") + 1 : -1].split("x"))
+        # Dimensions are padded/static; algorithmic FLOPs use the unpadded row count.
+        per_launch = 2 * rows * (n if "row_sparse" not in label else m) * (k if "row_sparse" not in label else n)
+        entry["tflops"] = round(per_launch / (ms * 1e-3) / 1e12, 1)
+        entry["frac_of_mfma_peak"] = round(entry["tflops"] / peak_tflops, 4)
+        entry["tflops_best"] = round(per_launch / (entry["ms_min"] * 1e-3) / 1e12, 1)
+    elif label in ("fm_copy_dense_to_sparse", "fm_copy_sparse_to_dense"):
+        work_bytes = workload.copy_bytes + rows * (index_size + 4)  # rows + indices + fp32 scores
+    elif label == "fm_copy_sparse_to_dense_backward":
+        work_bytes = (1 + 2 * workload.experts_per_token) * workload.tokens * hidden * itemsize
+    elif label.startswith("fm_mlp_activation"):
+        factor = 3 if label.endswith("forward") else (6 if recompute_level.recompute_activation else 5)
+        work_bytes = factor * rows * ffn * itemsize
+    if work_bytes is not None:
+        entry["gbs"] = round(work_bytes / (ms * 1e-3) / 1e9, 1)
+        entry["frac_of_hbm_peak"] = round(entry["gbs"] / PEAK_HBM_GBS, 4)
+        entry["gbs_best"] = round(work_bytes / (entry["ms_min"] * 1e-3) / 1e9, 1)
+    return entry
+
+
+def isolated_kernels(workload, inputs, device, recompute_level, repetitions: int = 20) -> dict:
+    """Every kernel of the step launched on its own, on the step's own operands, with the caches flushed before each
+    launch (a 512 MiB buffer is overwritten: twice the Infinity Cache, so operands and whatever an earlier kernel
+    left behind come from HBM): median and minimum of `repetitions` launches, HIP events around the library call.
+    The method of the reference's kernel benchmarks (tools/benchmark/triton_kernels/runner.py:211-276)."""
+    from fast_llm_amd import _lib
+    from fast_llm_amd.functional import sparse_copy, sparse_linear
+    from fast_llm_amd.functional.config import ActivationType
+    from fast_llm_amd.functional.mlp import mlp_activation_backward, mlp_activation_forward
+
+    silu = ActivationType.silu
+    x, scores, grad_output = inputs.hidden_states, inputs.scores, inputs.grad_output
+    weight_1, weight_2 = inputs.weight_1.detach(), inputs.weight_2.detach()
+    sparse_map = sparse_copy.get_sparse_map(inputs.top_experts, workload.experts)
+    # The operands of every kernel, computed once in the order of a step.
+    x_sparse = sparse_copy.copy_dense_to_sparse(x, None, sparse_map)
+    layer_1 = sparse_linear.output_sparse_matmul(x_sparse, weight_1.t(), sparse_map)
+    activation = mlp_activation_forward(layer_1, True, silu, sparse_map)[0]
+    layer_2 = sparse_linear.input_inner_sparse_matmul(activation, weight_2, sparse_map)
+    grad_layer_2 = sparse_copy.copy_sparse_to_dense_backward(grad_output, (sparse_map, layer_2, scores))[0]
+    grad_activation = sparse_linear.output_sparse_matmul(grad_layer_2, weight_2.t(), sparse_map)
+    grad_layer_1 = mlp_activation_backward(grad_activation, (layer_1, True, silu, sparse_map))[0]
+    grad_x_sparse = sparse_linear.input_inner_sparse_matmul(grad_layer_1, weight_1, sparse_map)
+    grad_weight_1, grad_weight_2 = torch.empty_like(weight_1), torch.empty_like(weight_2)
+    launches = [
+        lambda: sparse_copy.get_sparse_map(inputs.top_experts, workload.experts),
+        lambda: sparse_copy.copy_dense_to_sparse(x, None, sparse_map),
+        lambda: sparse_linear.output_sparse_matmul(x_sparse, weight_1.t(), sparse_map),
+        lambda: mlp_activation_forward(layer_1, True, silu, sparse_map),
+        lambda: sparse_linear.input_inner_sparse_matmul(activation, weight_2, sparse_map),
+        lambda: sparse_copy.copy_sparse_to_dense(layer_2, scores, sparse_map),
+        lambda: sparse_copy.copy_sparse_to_dense_backward(grad_output, (sparse_map, layer_2, scores)),
+        lambda: sparse_linear.output_sparse_matmul(grad_layer_2, weight_2.t(), sparse_map),
+        lambda: mlp_activation_backward(grad_activation, (layer_1, True, silu, sparse_map)),
+        lambda: sparse_linear.input_row_sparse_matmul(activation.t(), grad_layer_2, sparse_map, out=grad_weight_2),
+        lambda: sparse_linear.input_inner_sparse_matmul(grad_layer_1, weight_1, sparse_map),
+        lambda: sparse_linear.input_row_sparse_matmul(grad_layer_1.t(), x_sparse, sparse_map, out=grad_weight_1),
+    ]
+    flush = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=device)
+    durations: dict[str, list[float]] = {}
+    for launch in launches:
+        with _lib.KernelTimer() as timer:
+            for repetition in range(repetitions + 1):
+                flush.fill_(repetition & 0xFF)
+                launch()
+        for label, values in timer.durations_ms().items():
+            durations.setdefault(label, []).extend(values[1:])  # the first launch warms up
+    figures = {}
+    for label, values in sorted(durations.items()):
+        entry = kernel_figures(label, values, workload, recompute_level)
+        # Here the median is the figure: rate and fraction at the median instead of the mean.
+        for rate, peak_key in (("tflops", "frac_of_mfma_peak"), ("gbs", "frac_of_hbm_peak")):
+            if rate in entry:
+                entry[rate] = round(entry[rate] * entry["ms"] / entry["ms_median"], 1)
+                peak = PEAK_HBM_GBS if rate == "gbs" else (PEAK_FP32_TFLOPS if workload.dtype == torch.float32 else PEAK_BF16_TFLOPS)
+                entry[peak_key] = round(entry[rate] / peak, 4)
+        del entry["ms"]
+        figures[label] = entry
+    return {
+        "method": f"each kernel on its own, {FLUSH_BYTES >> 20} MiB overwritten before every launch, median and "
+        f"minimum of {repetitions} launches after one warm-up; rates and fractions at the median",
+        "kernels": figures,
+    }
+
+
+def graph_replay(timed: dict, device: torch.device, replays: int = 200) -> dict:
+    """The step captured once in a HIP graph and replayed: what is left of a launch-bound step when the host is out of
+    the way. The replayed step writes the same gradient as the eager one (checked)."""
+    step = timed["step"]
+    x = timed["state"][0]
+    step()
+    torch.cuda.synchronize()
+    eager_grad = x.grad.clone()
+    stream = torch.cuda.Stream(device=device)
+    stream.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(stream):
+        step()
+    torch.cuda.current_stream(device).wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    matches = bool(torch.equal(x.grad, eager_grad))
+    start = time.perf_counter()
+    for _ in range(replays):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - start) / replays * 1e3
+    return {"ms_per_step": round(ms, 4), "replays": replays, "matches_eager": matches}
 
 
 def summary_of(workload, timed: dict) -> dict:
@@ -223,15 +407,14 @@ def summary_of(workload, timed: dict) -> dict:
 
 
 def release(timed: dict) -> None:
-    timed.pop("inputs", None)
+    for key in ("inputs", "step", "state"):
+        timed.pop(key, None)
     torch.cuda.empty_cache()
 
 
 def measure_ceilings(device: torch.device) -> dict:
     """What the device sustains, for setting the kernels' figures against: see the module docstring."""
-    from fast_llm_amd import _lib
-
-    library = _lib.lib()
+    library = probes()
     stream = torch.cuda.current_stream(device)
     compute_units = torch.cuda.get_device_properties(device).multi_processor_count
 
@@ -249,11 +432,11 @@ def measure_ceilings(device: torch.device) -> dict:
     result: dict = {"compute_units": compute_units}
     sink = torch.empty(compute_units * 256, dtype=torch.float32, device=device)
     iterations = 40000  # about 30 ms per launch at the published peak
-    flops = library.fm_probe_mfma_flops(compute_units, iterations)
+    flops = library.probe_mfma_flops(compute_units, iterations)
     for name, random_operands, sigma in (("zeros", 0, 0.0), ("normal_sigma_0.02", 1, 0.02), ("normal_sigma_1", 1, 1.0)):
         ms = timed(
-            lambda: _lib.check(
-                library.fm_probe_mfma(sink.data_ptr(), compute_units, iterations, random_operands, sigma, stream.cuda_stream)
+            lambda: probe_ok(
+                library.probe_mfma(sink.data_ptr(), None, compute_units, iterations, random_operands, sigma, stream.cuda_stream)
             ),
             10,
         )
@@ -311,8 +494,8 @@ def measure_ceilings(device: torch.device) -> dict:
     target = torch.empty_like(source)
     for workgroups in (compute_units * 8, compute_units * 32, size // 16 // 256):
         ms = timed(
-            lambda: _lib.check(
-                library.fm_probe_copy(source.data_ptr(), target.data_ptr(), size, workgroups, stream.cuda_stream)
+            lambda: probe_ok(
+                library.probe_copy(source.data_ptr(), target.data_ptr(), size, workgroups, stream.cuda_stream)
             ),
             20,
         )
@@ -339,8 +522,8 @@ def measure_ceilings(device: torch.device) -> dict:
         groups = 8 * -(-(workgroups // 8) // shared_by)
         region = torch.empty(groups * region_bytes, dtype=torch.uint8, device=device).random_(0, 255)
         ms = timed(
-            lambda: _lib.check(
-                library.fm_probe_l2(
+            lambda: probe_ok(
+                library.probe_l2(
                     region.data_ptr(), region_bytes, shared_by, workgroups, iterations, in_flight, cycles.data_ptr(),
                     stream.cuda_stream,
                 )
@@ -439,8 +622,12 @@ def main() -> None:
         "kernels": timed["kernels"],
     }
     headline_inputs = timed["inputs"]
+    # Same run, same device, right after the timed steps: the MFMA rate and clock this box holds under load.
+    result["box"] = box_probe(device)
+    result["roofline"]["frac_of_box_mfma_loop"] = round(timed["gemm_tflops"] / result["box"]["mfma_loop_tflops_random"], 4)
 
     if not args.only:
+        result["isolated"] = isolated_kernels(workload, timed["inputs"], device, recompute_level)
         # The same step with the other gradient-buffer layout.
         other = "same" if args.grad_dtype == "fp32" else "fp32"
         headline_inputs = None if args.cpu_tokens <= 0 else timed["inputs"].to("cpu")
@@ -454,6 +641,19 @@ def main() -> None:
             "gemm_tflops": round(other_timed["gemm_tflops"], 1),
             "gemm_frac": round(other_timed["gemm_tflops"] / other_timed["gemm_peak_tflops"], 4),
         }
+        # The same step with full recomputation (layer 1 runs a second time in the backward; its forward takes the
+        # kernel with the activation in its epilogue, since its output is not stored).
+        if recompute_level != MLPRecomputeLevel.full:
+            full_timed = time_workload(workload, args, min(args.steps, 10), min(args.warmup, 2), args.grad_dtype,
+                                       MLPRecomputeLevel.full, device)  # fmt: skip
+            release(full_timed)
+            result["recompute_full"] = {
+                "ms_per_step": round(full_timed["ms_per_step"], 4),
+                "tokens_per_s": round(full_timed["tokens_per_s"], 1),
+                "gemm_tflops": round(full_timed["gemm_tflops"], 1),
+                "gemm_frac": round(full_timed["gemm_tflops"] / full_timed["gemm_peak_tflops"], 4),
+                "kernels": {label: entry["ms"] for label, entry in full_timed["kernels"].items()},
+            }
         # The other configurations: a few steps each, figures per configuration.
         configs = {workload.name: summary_of(workload, timed)}
         tiny_inputs = None
@@ -464,8 +664,17 @@ def main() -> None:
             config_timed = time_workload(other_workload, args, min(args.steps, 10), min(args.warmup, 2), "same",
                                          recompute_level, device)  # fmt: skip
             configs[name] = summary_of(other_workload, config_timed)
-            if name == "tiny" and args.cpu_tokens > 0:
-                tiny_inputs = config_timed["inputs"].to("cpu")
+            if name != "imbalanced":  # same shapes as the Mixtral-like configuration
+                isolated = isolated_kernels(other_workload, config_timed["inputs"], device, recompute_level)
+                configs[name]["isolated"] = {
+                    label: {key: value for key, value in entry.items() if key in _ISOLATED_KEYS}
+                    for label, entry in isolated["kernels"].items()
+                }
+            if name == "tiny":
+                # Launch-bound (a dozen kernels of 5 to 150 us per step): the step replayed from a HIP graph.
+                configs[name]["graph_replay"] = graph_replay(config_timed, device)
+                if args.cpu_tokens > 0:
+                    tiny_inputs = config_timed["inputs"].to("cpu")
             release(config_timed)
         result["configs"] = configs
         if tiny_inputs is not None:

@@ -13,7 +13,7 @@ import torch
 
 LIBRARY_PATH = pathlib.Path(__file__).resolve().parent / "csrc" / "libfastmoe_hip.so"
 
-FM_VERSION = 9
+FM_VERSION = 10
 
 _c_i64, _c_int, _c_ptr, _c_size = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
@@ -52,10 +52,6 @@ SIGNATURES: dict[str, tuple] = {
         _c_int,
         [_c_ptr] * 6 + [_c_i64] * 8 + [_c_int] * 3 + [_c_ptr],
     ),
-    "fm_probe_mfma": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_int, ctypes.c_float, _c_ptr]),
-    "fm_probe_mfma_flops": (_c_i64, [_c_i64, _c_i64]),
-    "fm_probe_copy": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
-    "fm_probe_l2": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),
 }
 
 FM_ERR_INVALID_ARGUMENT, FM_ERR_UNSUPPORTED, FM_ERR_LAUNCH = -1, -2, -3

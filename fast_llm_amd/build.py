@@ -49,19 +49,24 @@ def _compile(source: pathlib.Path) -> pathlib.Path:
     return obj
 
 
-def build_library(verbose: bool = True) -> pathlib.Path:
-    sources = sorted(CSRC.glob("*.hip"))
-    if not sources:
-        raise RuntimeError(f"no HIP sources in {CSRC}")
+def build_shared(sources: list[pathlib.Path], library: pathlib.Path, verbose: bool = True) -> pathlib.Path:
+    """Compile `sources` for gfx950 (in parallel) and link them into the shared library `library`."""
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         objects = list(pool.map(_compile, sources))
-    command = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objects), "-o", str(LIBRARY)]
+    command = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objects), "-o", str(library)]
     result = subprocess.run(command, capture_output=True, text=True)
     if result.returncode != 0:
         raise RuntimeError(f"link failed:\n{result.stderr}")
     if verbose:
-        print(f"built {LIBRARY} from {len(sources)} sources")
-    return LIBRARY
+        print(f"built {library} from {len(sources)} sources")
+    return library
+
+
+def build_library(verbose: bool = True) -> pathlib.Path:
+    sources = sorted(CSRC.glob("*.hip"))
+    if not sources:
+        raise RuntimeError(f"no HIP sources in {CSRC}")
+    return build_shared(sources, LIBRARY, verbose)
 
 
 if __name__ == "__main__":

@@ -601,10 +601,20 @@ __device__ __forceinline__ bool compute_tile_record(const GemmArgs &args, int id
     return true;
 }
 
-// One wavefront per id.
+// The 64 bytes in front of the records: how the launch splits its last round, for the kernel that adds the pieces.
+struct alignas(64) TableHeader {
+    SplitPlan plan;
+};
+static_assert(sizeof(TableHeader) == 64 && sizeof(TableHeader) == sizeof(TileRecord), "the header is record -1");
+
+// One wavefront per id; the wavefront of id 0 also leaves the split plan of the launch in the table's header.
 __global__ __launch_bounds__(256) void grouped_gemm_plan_kernel(GemmArgs args, TileRecord *table) {
     const int id = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (id >= args.num_ids) return;
+    if (id == 0 && args.partials != nullptr) {
+        const SplitPlan plan = plan_split(args);
+        if ((threadIdx.x & 63) == 0) reinterpret_cast<TableHeader *>(table)[-1].plan = plan;
+    }
     TileRecord record;
     record.unused[0] = record.unused[1] = 0;
     if (!compute_tile_record(args, id, record)) {
@@ -1287,7 +1297,8 @@ constexpr int kReduceLdsBytes = kWaves * 32 * (kWaveCols * 4 + kEpiloguePadBytes
 __global__ __launch_bounds__(64) void grouped_gemm_reduce_kernel(GemmArgs args) {
     extern __shared__ __attribute__((aligned(1024))) char lds_generic[];
     FM_LDS(char) *lds = (FM_LDS(char) *)(lds_generic);
-    const SplitPlan plan = plan_split(args);
+    // The plan kernel has left the split plan of this launch in front of the tile records.
+    const SplitPlan plan = static_cast<const TableHeader *>(args.tile_table)[-1].plan;
     const int index = blockIdx.x / kWaves;
     if (plan.pieces == 1 || index >= plan.tail) return;
     TileWork work;
@@ -1343,7 +1354,8 @@ static int launch_instance(const GemmArgs &args, hipStream_t stream) {
     auto kernel = grouped_gemm_mfma_kernel<T, kLhsK, kRhsK, kMasked, kFusion>;
     static std::atomic<uint64_t> configured{0};
     if (int status = allow_lds(reinterpret_cast<const void *>(kernel), kLdsBytes, configured)) return status;
-    // With a workspace, one wavefront per id first writes the id's tile record.
+    // With a workspace, one wavefront per id first writes the id's tile record (and, when the last round may be
+    // split, the plan of the split).
     if (args.tile_table != nullptr)
         grouped_gemm_plan_kernel<<<(args.num_ids + 3) / 4, 256, 0, stream>>>(args, static_cast<TileRecord *>(args.tile_table));
     // One workgroup per CU walks the ids (see the kernel).
@@ -1444,10 +1456,16 @@ static int count_ids(const GemmArgs &args, bool split) {
 }
 
 constexpr size_t kPartialBytes = sizeof(float) * kPartialFloats * kMaxPartials;
-static size_t table_bytes(int num_ids) { return (static_cast<size_t>(num_ids) * sizeof(TileRecord) + 255) / 256 * 256; }
+// The header, then one record per id.
+static size_t table_bytes(int num_ids) {
+    return (sizeof(TableHeader) + static_cast<size_t>(num_ids) * sizeof(TileRecord) + 255) / 256 * 256;
+}
 
 size_t mfma_gemm_workspace_size(GemmArgs args) {
     if (args.rows <= 0 || args.cols <= 0 || args.inner <= 0) return 0;
+    // Dimensions that `mfma_gemm_eligible` refuses whatever the strides: such a product runs on the generic kernel,
+    // which takes no workspace.
+    if (args.inner % kBK != 0 || args.cols % 8 != 0 || (args.mode == kInputRowSparse && args.sparse_size % 8 != 0)) return 0;
     count_tiles(args);
     if (too_many_tiles(args)) return 0;
     const bool split = splits_last_round(args);
@@ -1468,7 +1486,10 @@ int mfma_gemm_launch(GemmArgs args, int dtype, void *workspace, size_t workspace
                         "grouped gemm: workspace of %zu bytes (64-byte aligned) needed, got %zu at %p", needed,
                         workspace_size, workspace);
         if (split) args.partials = static_cast<float *>(workspace);
-        args.tile_table = static_cast<char *>(workspace) + (split ? kPartialBytes : 0);
+        args.tile_table = static_cast<char *>(workspace) + (split ? kPartialBytes : 0) + sizeof(TableHeader);
+        // A launch of at most one round that does not split: every workgroup finds its one tile itself (a scan of the
+        // expert map, a few thousand cycles) sooner than a kernel launched in front of it could tell it.
+        if (!split && args.num_ids <= kRound) args.tile_table = nullptr;
     }
     return dtype == FM_DTYPE_BF16 ? launch_layout<bf16_t>(args, stream) : launch_layout<f16_t>(args, stream);
 }

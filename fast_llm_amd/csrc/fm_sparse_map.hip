@@ -168,15 +168,17 @@ __global__ __launch_bounds__(kMapBlock) void sparse_map_rows_kernel(const int64_
                                                                     const int32_t *__restrict__ block_prefix,
                                                                     const int32_t *__restrict__ expert_begins,
                                                                     int index_dtype, void *__restrict__ sparse_rows) {
-    extern __shared__ int32_t lds_map[];  // [kMapWaves][num_experts] counts per wavefront, then [num_experts] running
-    int32_t *lds_wave_counts = lds_map;
-    int32_t *lds_running = lds_map + kMapWaves * num_experts;
+    static_assert(kMapMaxExperts <= kMapBlock, "thread e keeps the running count of expert e in a register");
+    extern __shared__ int32_t lds_wave_counts[];  // [kMapWaves][num_experts] counts per wavefront: 64 KiB at 1024 experts
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int num_bits = log2_ceil(num_experts);
     const int64_t first = static_cast<int64_t>(blockIdx.x) * entries_per_block;
     const int64_t last = min(first + entries_per_block, num_entries);
-    for (int e = threadIdx.x; e < num_experts; e += kMapBlock)
-        lds_running[e] = expert_begins[e] + block_prefix[static_cast<int64_t>(blockIdx.x) * num_experts + e];
+    // Rows handed out so far to expert threadIdx.x (there are at most as many experts as threads).
+    const int own_expert = threadIdx.x;
+    int32_t running = 0;
+    if (own_expert < num_experts)
+        running = expert_begins[own_expert] + block_prefix[static_cast<int64_t>(blockIdx.x) * num_experts + own_expert];
 
     for (int64_t chunk = first; chunk < last; chunk += kMapBlock) {
         for (int i = threadIdx.x; i < kMapWaves * num_experts; i += kMapBlock) lds_wave_counts[i] = 0;
@@ -192,15 +194,13 @@ __global__ __launch_bounds__(kMapBlock) void sparse_map_rows_kernel(const int64_
         __syncthreads();
 
         // Exclusive prefix over the wavefronts of the workgroup, per expert, in place, on top of the running count.
-        for (int e = threadIdx.x; e < num_experts; e += kMapBlock) {
-            int32_t running = lds_running[e];
+        if (own_expert < num_experts) {
 #pragma unroll
             for (int w = 0; w < kMapWaves; ++w) {
-                const int32_t here = lds_wave_counts[w * num_experts + e];
-                lds_wave_counts[w * num_experts + e] = running;
+                const int32_t here = lds_wave_counts[w * num_experts + own_expert];
+                lds_wave_counts[w * num_experts + own_expert] = running;
                 running += here;
             }
-            lds_running[e] = running;
         }
         __syncthreads();
 
@@ -245,7 +245,7 @@ static int run_sparse_map(const char *name, const int64_t *top_experts, int64_t 
     sparse_map_layout_kernel<<<1, kMapBlock, 0, stream>>>(block_counts, blocks, experts, pad_to_multiple, index_dtype,
                                                           expert_ends, expert_pad_begins, expert_begins);
     if (blocks > 0) {
-        sparse_map_rows_kernel<<<blocks, kMapBlock, (kMapWaves + 1) * experts * sizeof(int32_t), stream>>>(
+        sparse_map_rows_kernel<<<blocks, kMapBlock, kMapWaves * experts * sizeof(int32_t), stream>>>(
             top_experts, num_entries, kMapBlock, experts, block_counts, expert_begins, index_dtype, sparse_rows);
     }
     return check_launch(name);
@@ -329,7 +329,7 @@ extern "C" int fm_sparse_map_from_router(const int64_t *top_experts, const void 
         static_cast<const float *>(router_workspace), stats, blocks, num_tokens, tokens_per_block,
         static_cast<int>(routed), experts, pad_to_multiple, index_dtype, expert_ends, expert_pad_begins, block_prefix,
         expert_begins);
-    sparse_map_rows_kernel<<<blocks, kMapBlock, (kMapWaves + 1) * experts * sizeof(int32_t), stream>>>(
+    sparse_map_rows_kernel<<<blocks, kMapBlock, kMapWaves * experts * sizeof(int32_t), stream>>>(
         top_experts, num_tokens * slots, tokens_per_block * slots, experts, block_prefix, expert_begins, index_dtype,
         sparse_rows);
     return check_launch(name);
@@ -347,12 +347,20 @@ constexpr int kMaxDevices = 64;
 
 // Device address of this device's copy of `scratch`, looked up once per device with that device current. In host
 // code the array's name is not a device address; only the pointer returned here may go to kernels.
-static int static_scratch_of_current_device(void **pointer) {
+// `stream` (may be null: the current device's default stream) must belong to the current device: the kernels run where
+// the stream lives, and each device has its own copy of the array.
+static int static_scratch_of_current_device(hipStream_t stream, void **pointer) {
     static std::mutex mutex;
     static void *addresses[kMaxDevices] = {};
     int device = -1;
     hipError_t error = hipGetDevice(&device);
     if (error != hipSuccess) return fail(FM_ERR_LAUNCH, "fm_sparse_map_static: hipGetDevice: %s", hipGetErrorString(error));
+    int stream_device = device;
+    if (stream != nullptr && hipStreamGetDevice(stream, &stream_device) == hipSuccess && stream_device != device)
+        return fail(FM_ERR_INVALID_ARGUMENT,
+                    "fm_sparse_map_static: the stream belongs to device %d but device %d is current; make the stream's "
+                    "device current before the call",
+                    stream_device, device);
     if (device < 0 || device >= kMaxDevices)
         return fail(FM_ERR_UNSUPPORTED, "fm_sparse_map_static: device %d outside [0, %d)", device, kMaxDevices);
     std::lock_guard<std::mutex> lock(mutex);
@@ -387,7 +395,7 @@ extern "C" int fm_sparse_map_static(const int64_t *top_experts, int64_t num_rows
                     (long long)num_rows_dense, (long long)num_experts_per_token, (long long)num_experts, needed,
                     kStaticScratchBytes);
     void *workspace = nullptr;
-    if (int status = static_scratch_of_current_device(&workspace)) return status;
+    if (int status = static_scratch_of_current_device(static_cast<hipStream_t>(stream), &workspace)) return status;
     // Nothing to clear: the histogram kernel writes every count the other two kernels read.
     return run_sparse_map("fm_sparse_map_static", top_experts, num_rows_dense, num_experts_per_token, num_experts,
                           pad_to_multiple, index_dtype, sparse_rows, expert_ends, expert_pad_begins, workspace,

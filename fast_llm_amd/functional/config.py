@@ -17,14 +17,15 @@ class KernelConfig:
     """
 
     POINTWISE_BLOCK_SIZE = 1024
-    # Run a gated sparse MLP's activation (forward and backward) in the epilogue of the neighbouring grouped product
-    # when the shapes allow. Results are bit-identical either way. Off by default: measured slower on MI355X at the
-    # Mixtral shape (layer 1 forward 3.45 ms fused against 3.06 + 0.24 ms separate, layer 2 input gradient 2.15 ms
-    # against 1.56 + 0.40 ms). The matrix-core kernel runs one wavefront per SIMD, so the exponentials and
-    # reciprocals of the epilogue run with nothing to overlap them, while the separate streaming kernel does the
-    # same arithmetic at full occupancy behind its memory traffic. It pays only where layer 1's output is not
-    # stored at all (inference, full recomputation: 3.27 ms against 3.14 + 0.24 ms).
-    fuse_activation = False
+    # Whether a gated sparse MLP's activation runs in the epilogue of the neighbouring grouped product (layer 1 forward;
+    # layer 2 input gradient) where the shapes allow. Results are bit-identical either way. None (default): chosen per
+    # call, fused exactly where it was measured faster on MI355X, which is the layer 1 forward whose own output is not
+    # stored (inference, `MLPRecomputeLevel.full`: 3.27 ms against 3.14 + 0.24 ms at the Mixtral shape). Where layer
+    # 1's output is kept the fused kernels are slower (forward 3.45 ms against 3.06 + 0.24 ms, layer 2 input gradient
+    # 2.15 ms against 1.56 + 0.40 ms): the matrix-core kernel runs one wavefront per SIMD, so the exponentials and
+    # reciprocals of the epilogue run with nothing to overlap them, while the separate streaming kernel does the same
+    # arithmetic at full occupancy behind its memory traffic. True: fuse both wherever possible; False: never.
+    fuse_activation: bool | None = None
     # Hand the grouped products their scratch: a table of where every tile of a launch lies, written by a small
     # kernel before the product (the product's workgroups then look their tiles up instead of each scanning the expert
     # map), and the space with which a launch of few, long tiles (layer 2 forward and the layer 1 input gradient at

@@ -196,6 +196,52 @@ def gated_layer_2_input_backward(
     return grad_layer_1, output
 
 
+class _MLPContext(typing.NamedTuple):
+    """What `mlp_forward` hands `mlp_backward`, in the positional layout of the reference's context list
+    (fast_llm/functional/triton/mlp.py:287-306). An intermediate that the recompute level does not keep is None."""
+
+    input_: torch.Tensor | None  # dense tokens; kept only when the sparse copy of them is recomputed
+    scores: torch.Tensor | None
+    sparse_input: torch.Tensor | None  # tokens in the expert-sorted layout (the dense input itself without a map)
+    layer_1_output: torch.Tensor | None
+    activation_output: torch.Tensor | None
+    layer_2_output: torch.Tensor | None  # always kept with a map: the score gradient reads it
+    weight_1: torch.Tensor
+    bias_1: torch.Tensor | None
+    weight_2: torch.Tensor
+    bias_2: torch.Tensor | None
+    gated: bool
+    activation_type: ActivationType
+    group: typing.Any
+    sequence_parallel: bool
+    transposed_layer_2_weight: bool
+    sparse_map: SparseMap | None
+    input_shape: torch.Size
+    use_triton: bool | None
+
+
+def _fuse_forward(keep_layer_1: bool) -> bool:
+    """Whether layer 1 takes the kernel with the activation in its epilogue: when asked to, and by default exactly
+    where that kernel wins, i.e. where layer 1's output is not stored (see `KernelConfig.fuse_activation`)."""
+    return not keep_layer_1 if KernelConfig.fuse_activation is None else bool(KernelConfig.fuse_activation)
+
+
+def _fuse_backward() -> bool:
+    return bool(KernelConfig.fuse_activation)  # by default never: measured slower than the two kernels
+
+
+def _layer_1_and_activation(sparse_input, weight_1, bias_1, gated, activation_type, sparse_map, keep_layer_1):
+    """(layer-1 output or None if it is neither kept nor needed, activation output)."""
+    if _fuse_forward(keep_layer_1) and _fusable(sparse_input, weight_1.t(), gated, sparse_map, bias_1):
+        try:
+            return gated_layer_1_forward(sparse_input, weight_1, sparse_map, activation_type, keep_layer_1)
+        except NotImplementedError:  # a shape the fused kernel does not tile
+            pass
+    layer_1_output, _ = output_parallel_linear_forward(sparse_input, weight_1, bias_1, None, False, False, True, sparse_map)
+    activation_output, _ = mlp_activation_forward(layer_1_output, gated, activation_type, sparse_map)
+    return (layer_1_output if keep_layer_1 else None), activation_output
+
+
 def mlp_forward(
     input_: torch.Tensor,
     scores: torch.Tensor | None,
@@ -221,74 +267,44 @@ def mlp_forward(
     if group is not None or sequence_parallel:
         raise NotImplementedError("tensor/sequence parallelism is not part of this single-GPU path")
     KernelConfig.enabled(input_.device, use_triton)
+    sparse = sparse_map is not None
+    keep_layer_1 = training and not recompute_level.recompute_layer_1
+    keep_activation = training and not recompute_level.recompute_activation
 
-    # Sparse copy
-    input_shape = input_.shape
-    intermediate_0 = input_ if sparse_map is None else copy_dense_to_sparse_forward(input_, sparse_map)[0]
-
-    # Layer 1 and activation: one kernel where the library has one, else the reference's two steps.
-    intermediate_2 = None
-    if KernelConfig.fuse_activation and _fusable(intermediate_0, weight_1.t(), gated, sparse_map, bias_1):
-        try:
-            intermediate_1, intermediate_2 = gated_layer_1_forward(
-                intermediate_0, weight_1, sparse_map, activation_type, training and not recompute_level.recompute_layer_1
-            )
-        except NotImplementedError:
-            pass
-    if intermediate_2 is None:
-        intermediate_1, _ = output_parallel_linear_forward(
-            intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
-        )
-        intermediate_2, _ = mlp_activation_forward(intermediate_1, gated, activation_type, sparse_map)
-
-    if recompute_level.recompute_sparse_input:
-        intermediate_0 = None
-    else:
-        input_ = None
-    if recompute_level.recompute_layer_1:
-        intermediate_1 = None
-
-    # Layer 2
-    intermediate_3, _ = input_parallel_linear_forward(
-        intermediate_2, weight_2, bias_2, group, False, transposed_layer_2_weight, True, sparse_map
+    sparse_input = copy_dense_to_sparse_forward(input_, sparse_map)[0] if sparse else input_
+    layer_1_output, activation_output = _layer_1_and_activation(
+        sparse_input, weight_1, bias_1, gated, activation_type, sparse_map, keep_layer_1
     )
-
-    # Context
-    if recompute_level.recompute_activation or not training:
-        intermediate_2 = None
-
-    # Sparse copy
-    if sparse_map is None:
-        output = intermediate_3
-        intermediate_3 = None
-    else:
-        output, _ = copy_sparse_to_dense_forward(intermediate_3, scores, sparse_map)
-
-    context = (
-        [
-            input_,
-            scores,
-            intermediate_0,
-            intermediate_1,
-            intermediate_2,
-            intermediate_3,
-            weight_1,
-            bias_1,
-            weight_2,
-            bias_2,
-            gated,
-            activation_type,
-            group,
-            sequence_parallel,
-            transposed_layer_2_weight,
-            sparse_map,
-            input_shape,
-            use_triton,
-        ]
-        if training
-        else None
+    layer_2_output, _ = input_parallel_linear_forward(
+        activation_output, weight_2, bias_2, group, False, transposed_layer_2_weight, True, sparse_map
     )
-    return output, context
+    output = copy_sparse_to_dense_forward(layer_2_output, scores, sparse_map)[0] if sparse else layer_2_output
+    if not training:
+        return output, None
+
+    # Either the dense tokens or their sparse copy go to the backward, never both.
+    recompute_input = recompute_level.recompute_sparse_input
+    context = _MLPContext(
+        input_=input_ if recompute_input else None,
+        scores=scores,
+        sparse_input=None if recompute_input else sparse_input,
+        layer_1_output=layer_1_output,
+        activation_output=activation_output if keep_activation else None,
+        layer_2_output=layer_2_output if sparse else None,
+        weight_1=weight_1,
+        bias_1=bias_1,
+        weight_2=weight_2,
+        bias_2=bias_2,
+        gated=gated,
+        activation_type=activation_type,
+        group=group,
+        sequence_parallel=sequence_parallel,
+        transposed_layer_2_weight=transposed_layer_2_weight,
+        sparse_map=sparse_map,
+        input_shape=input_.shape,
+        use_triton=use_triton,
+    )
+    return output, list(context)
 
 
 def mlp_backward(grad_output: torch.Tensor, context: list[typing.Any]) -> tuple[torch.Tensor, torch.Tensor]:
@@ -296,87 +312,66 @@ def mlp_backward(grad_output: torch.Tensor, context: list[typing.Any]) -> tuple[
     Backward of `mlp_forward`: returns (grad_input, grad_scores); weight gradients go to the grad buffers.
     Reference: fast_llm/functional/triton/mlp.py:314-415.
     """
-    (
-        input_,
-        scores,
-        intermediate_0,
-        intermediate_1,
-        intermediate_2,
-        intermediate_3,
-        weight_1,
-        bias_1,
-        weight_2,
-        bias_2,
-        gated,
-        activation_type,
-        group,
-        sequence_parallel,
-        transposed_layer_2_weight,
-        sparse_map,
-        input_shape,
-        use_triton,
-    ) = context
-    context.clear()
+    saved = _MLPContext(*context)
+    context.clear()  # the list may outlive this call (autograd holds it): let go of the tensors now
+    sparse_map, gated, activation_type = saved.sparse_map, saved.gated, saved.activation_type
+    weight_2, bias_2, transposed_layer_2_weight = saved.weight_2, saved.bias_2, saved.transposed_layer_2_weight
+    input_shape = saved.input_shape
+    sparse = sparse_map is not None
 
-    # Sparse copy
-    if sparse_map is None:
-        grad_scores = None
-    else:
-        grad_output, grad_scores = copy_sparse_to_dense_backward(grad_output, (sparse_map, intermediate_3, scores))
+    # Backward of the combine: the gradient of layer 2's output, and of the scores.
+    grad_scores = None
+    if sparse:
+        grad_output, grad_scores = copy_sparse_to_dense_backward(
+            grad_output, (sparse_map, saved.layer_2_output, saved.scores)
+        )
 
-    # Sparse input recomputation
-    if intermediate_0 is None:
-        intermediate_0 = input_ if sparse_map is None else copy_dense_to_sparse_forward(input_, sparse_map)[0]
+    # Whatever the forward did not keep is computed again, front to back.
+    sparse_input = saved.sparse_input
+    if sparse_input is None:
+        sparse_input = copy_dense_to_sparse_forward(saved.input_, sparse_map)[0] if sparse else saved.input_
+    layer_1_context = (sparse_input, saved.weight_1, saved.bias_1, None, False, False, True, sparse_map)
+    layer_1_output = saved.layer_1_output
+    if layer_1_output is None:
+        layer_1_output = output_parallel_linear_forward(*layer_1_context)[0]
+    activation_output = saved.activation_output
+    recompute_activation = activation_output is None
+    del saved  # every intermediate now has one name here and is released as soon as its last reader is done
 
-    # Layer 1 recomputation
-    if intermediate_1 is None:
-        intermediate_1 = output_parallel_linear_forward(
-            intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map
-        )[0]
-
-    # Layer 2 input grad, then activation recomputation and/or backward: in one kernel where the library has one
-    # (the reference computes the layer 2 input grad before the two recomputations; they are independent).
+    # Gradient of layer 1's output = activation backward of (grad_output x W2^T), which also recomputes the
+    # activation output if needed: one kernel where the library has one and is asked to use it, else two. (The
+    # reference takes the layer-2 input gradient before its recomputations; the order does not matter.)
     weight_2_t = maybe_transpose(weight_2, transposed_layer_2_weight)
-    grad_intermediate_1 = None
-    if KernelConfig.fuse_activation and _fusable(grad_output, weight_2_t, gated, sparse_map):
+    grad_layer_1_output = None
+    if _fuse_backward() and _fusable(grad_output, weight_2_t, gated, sparse_map):
         try:
-            grad_intermediate_1, intermediate_2_ = gated_layer_2_input_backward(
-                grad_output, weight_2_t, sparse_map, intermediate_1, activation_type, intermediate_2 is None
+            grad_layer_1_output, recomputed = gated_layer_2_input_backward(
+                grad_output, weight_2_t, sparse_map, layer_1_output, activation_type, recompute_activation
             )
         except NotImplementedError:
             pass
-    if grad_intermediate_1 is None:
-        if sparse_map is None:
-            grad_intermediate_2 = grad_output.matmul(weight_2_t)
+    if grad_layer_1_output is None:
+        if sparse:
+            grad_activation_output = output_sparse_matmul(grad_output, weight_2_t, sparse_map)
         else:
-            grad_intermediate_2 = output_sparse_matmul(grad_output, weight_2_t, sparse_map)
-        grad_intermediate_1, intermediate_2_ = mlp_activation_backward(
-            grad_intermediate_2.contiguous(), (intermediate_1, gated, activation_type, sparse_map), intermediate_2 is None
+            grad_activation_output = grad_output.matmul(weight_2_t)
+        grad_layer_1_output, recomputed = mlp_activation_backward(
+            grad_activation_output.contiguous(), (layer_1_output, gated, activation_type, sparse_map), recompute_activation
         )
-        del grad_intermediate_2
+        del grad_activation_output
+    del layer_1_output
+    if recompute_activation:
+        activation_output = recomputed
+    del recomputed
 
-    # Layer 2 parameter grad
-    del intermediate_1
-    update_linear_gradients(
-        intermediate_2_ if intermediate_2 is None else intermediate_2,
-        weight_2,
-        bias_2,
-        grad_output,
-        transposed_layer_2_weight,
-        sparse_map,
-    )
-    del grad_output, intermediate_2, intermediate_2_
+    # Layer 2's weight gradient, then layer 1's input and weight gradients.
+    update_linear_gradients(activation_output, weight_2, bias_2, grad_output, transposed_layer_2_weight, sparse_map)
+    del grad_output, activation_output
+    grad_input = output_parallel_linear_backward(grad_layer_1_output, layer_1_context)
 
-    # Layer 1 backward
-    grad_input = output_parallel_linear_backward(
-        grad_intermediate_1,
-        (intermediate_0, weight_1, bias_1, group, False, False, True, sparse_map),
-    )
-
-    # Sparse copy
-    if sparse_map is not None:
+    # Backward of the dispatch.
+    if sparse:
         grad_input = copy_dense_to_sparse_backward(grad_input, (sparse_map, input_shape))
-
     return grad_input, grad_scores
 
 

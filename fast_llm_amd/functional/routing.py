@@ -23,6 +23,14 @@ class RouterCounts:
     routed_experts: int
     experts_per_token: int
     shared_experts: int
+    # Identity of the `top_experts` tensor the counts belong to (its storage address and in-place version counter):
+    # counts of other, or since edited, selections would give overlapping expert ranges.
+    top_experts_address: int = 0
+    top_experts_version: int = -1
+
+    def describes(self, top_experts: torch.Tensor) -> bool:
+        """Whether `top_experts` is the very tensor these counts were taken from, unmodified since."""
+        return top_experts.data_ptr() == self.top_experts_address and top_experts._version == self.top_experts_version
 
 
 def topk_routing_forward(logits: torch.Tensor, experts_per_token: int) -> tuple[torch.Tensor, torch.Tensor]:
@@ -131,7 +139,9 @@ def router_forward(
         shared_experts,
         _lib.dtype_tag(logits.dtype),
     )
-    counts = RouterCounts(workspace, tokens, experts, experts_per_token, shared_experts)
+    counts = RouterCounts(
+        workspace, tokens, experts, experts_per_token, shared_experts, top_experts.data_ptr(), top_experts._version
+    )
     return scores, top_experts, losses, lse, statistics, counts
 
 
@@ -206,7 +216,12 @@ def router(
     shape = logits.shape[:-1] + (shared_experts + experts_per_token,)
     result = (scores.view(shape), top_experts.view(shape), losses[0], losses[1])
     if return_counts:
-        result += (RouterCounts(workspace, flat.size(0), flat.size(1), experts_per_token, shared_experts),)
+        result += (
+            RouterCounts(
+                workspace, flat.size(0), flat.size(1), experts_per_token, shared_experts,
+                top_experts.data_ptr(), top_experts._version,
+            ),
+        )  # fmt: skip
     return result
 
 

@@ -50,7 +50,8 @@ def get_sparse_map(
     has no effect here; `use_triton=False` selects the reference's torch path, which this package does not have).
     `router_counts` (not in the reference's signature): the `RouterCounts` that `functional.routing.router` returned
     together with these very `top_experts`; the map is then built from the router's counts, without the pass that
-    counts `top_experts`. Same result.
+    counts `top_experts`. Same result. Counts that belong to another tensor, or to one modified in place since the
+    routing (masking, capacity or dropping hooks), are not used: the map then counts `top_experts` itself.
     """
     KernelConfig.enabled(top_experts.device, use_triton)
     Assert.eq(top_experts.dim(), 2)
@@ -60,6 +61,8 @@ def get_sparse_map(
     max_rows = (num_rows_unpadded + num_experts * pad_to_multiple) // pad_to_multiple * pad_to_multiple
     dtype = torch.int16 if max_rows < 32768 else torch.int32
 
+    if router_counts is not None and not router_counts.describes(top_experts):
+        router_counts = None
     top_experts = top_experts.to(torch.int64).contiguous()
     sparse_rows = torch.empty((num_rows_dense, num_experts_per_token), dtype=dtype, device=device)
     expert_ends = torch.empty(num_experts, dtype=dtype, device=device)
@@ -89,7 +92,6 @@ def get_sparse_map(
             _lib.ptr(expert_pad_begins),
             _lib.ptr(workspace),
             workspace_size,
-            label="fm_sparse_map",
         )
         return _finish_sparse_map(
             sparse_rows, expert_ends, expert_pad_begins, num_experts, dynamic_shape, max_rows

@@ -84,7 +84,6 @@ class DroplessMoEMLP(torch.nn.Module):
         )
         self.gated, self.activation = gated, activation
         self.recompute_level, self.dropless_dynamic_shape = recompute_level, dropless_dynamic_shape
-        self._router_counts = None
         layer_1_rows = experts * intermediate_size * (2 if gated else 1)
         self.router = torch.nn.Parameter(torch.empty(self.unshared_experts, hidden_size, dtype=dtype, device=device))
         self.layer_1 = torch.nn.Parameter(torch.empty(layer_1_rows, hidden_size, dtype=dtype, device=device))
@@ -104,6 +103,13 @@ class DroplessMoEMLP(torch.nn.Module):
         """Router logits to (scores, top_experts), shared experts included. `grad_scale` (the reference's
         `kwargs["grad_output"]`) makes the two auxiliary losses train the router; `losses` collects their values
         (mixture_of_experts.py:146-171, 237-262)."""
+        return self.route_with_counts(hidden_states, grad_scale, losses)[:2]
+
+    def route_with_counts(
+        self, hidden_states: torch.Tensor, grad_scale: float | None = None, losses: dict | None = None
+    ) -> tuple:
+        """`route`, followed by what the router's kernel counted on its way (the `RouterCounts` for `get_sparse_map`
+        together with the returned `top_experts`; None for sinkhorn routing, which does not count)."""
         router_input = hidden_states if self.router_normalization is None else self.router_normalization(hidden_states)
         if self.router_scale is not None:
             router_input = router_input * self.router_scale
@@ -115,8 +121,9 @@ class DroplessMoEMLP(torch.nn.Module):
             noise = torch.empty_like(logits).uniform_(1.0 - self.jitter_eps, 1.0 + self.jitter_eps)
         trained = self.training and grad_scale is not None
         if self.routing == ROUTING_SINKHORN:
-            return self._scale_per_expert(*self._route_sinkhorn(logits, noise, grad_scale if trained else None, losses))
-        scores, top_experts, load_balancing_loss, z_loss, self._router_counts = router(
+            routed = self._route_sinkhorn(logits, noise, grad_scale if trained else None, losses)
+            return (*self._scale_per_expert(*routed), None)
+        scores, top_experts, load_balancing_loss, z_loss, router_counts = router(
             logits,
             self.experts_per_token,
             shared_experts=self.shared_experts,
@@ -129,7 +136,7 @@ class DroplessMoEMLP(torch.nn.Module):
             losses.setdefault(LOAD_BALANCING_LOSS, []).append(load_balancing_loss)
             if self.z_loss_coefficient > 0.0:
                 losses.setdefault(ROUTER_Z_LOSS, []).append(z_loss)
-        return self._scale_per_expert(scores, top_experts)
+        return (*self._scale_per_expert(scores, top_experts), router_counts)
 
     def _scale_per_expert(self, scores: torch.Tensor, top_experts: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         if self.router_per_expert_scale is not None:  # mixture_of_experts.py:174-175
@@ -140,7 +147,6 @@ class DroplessMoEMLP(torch.nn.Module):
         self, logits: torch.Tensor, noise: torch.Tensor | None, grad_scale: float | None, losses: dict | None
     ) -> tuple[torch.Tensor, torch.Tensor]:
         """z-loss, jitter and sinkhorn routing as the reference orders them (mixture_of_experts.py:146-171)."""
-        self._router_counts = None
         if self.z_loss_coefficient > 0.0 and (grad_scale is not None or losses is not None):
             loss = torch.mean(torch.logsumexp(logits.float(), dim=-1) ** 2)
             if losses is not None:
@@ -164,9 +170,8 @@ class DroplessMoEMLP(torch.nn.Module):
         hidden_states = input_.flatten(0, -2)
         router_counts = None
         if top_experts is None:
-            scores, top_experts = self.route(hidden_states, grad_scale, losses)
             # The router has counted the tokens of every expert on its way: the map need not count them again.
-            router_counts, self._router_counts = self._router_counts, None
+            scores, top_experts, router_counts = self.route_with_counts(hidden_states, grad_scale, losses)
         sparse_map = get_sparse_map(
             top_experts, self.experts, dynamic_shape=self.dropless_dynamic_shape, router_counts=router_counts
         )

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define FM_VERSION 9
+#define FM_VERSION 10
 
 /* Element type of activations, weights and outputs. */
 enum fm_dtype { FM_DTYPE_F32 = 0, FM_DTYPE_BF16 = 1, FM_DTYPE_F16 = 2 };
@@ -100,7 +100,9 @@ int fm_sparse_map(const int64_t *top_experts,   /* [num_rows_dense, num_experts_
  * with FM_ERR_UNSUPPORTED (1 MiB covers e.g. 131072 x 8 entries over 128 experts, or 16384 x 8 over 1024). All calls
  * on one GPU share that GPU's array: calls that may overlap (different streams, different threads) race; calls on one
  * stream are safe. The array's address is looked up at a device's first call (a host-side query, no allocation); make
- * that first call outside graph capture. */
+ * that first call outside graph capture. The device the stream belongs to must be the current device (the array is
+ * looked up for the current device and the kernels run where the stream lives): a stream of another device is
+ * FM_ERR_INVALID_ARGUMENT. */
 #define FM_SPARSE_MAP_STATIC_SCRATCH_BYTES (1 << 20)
 size_t fm_sparse_map_static_scratch_size(void);
 int fm_sparse_map_static(const int64_t *top_experts, int64_t num_rows_dense, int64_t num_experts_per_token,
@@ -200,6 +202,9 @@ int fm_router_backward(const void *grad_scores, const void *scores, const void *
  * (same num_tokens; num_experts here counts routed + shared experts), this builds the map of `top_experts`
  * [num_tokens, shared_experts + experts_per_token] without the counting pass over `top_experts`. Same results as
  * `fm_sparse_map(top_experts, num_tokens, shared_experts + experts_per_token, num_experts, ...)`, bit for bit.
+ * Precondition (not checked, the counts are trusted): `top_experts` is exactly what that `fm_router_forward` call
+ * wrote. Selections edited since (masking, capacity or dropping) or counts of another call give expert ranges that
+ * overlap or run past `expert_ends`; rebuild the map with `fm_sparse_map` then.
  * Replaces the same reference lines as `fm_sparse_map`, for the caller
  * fast_llm/layers/decoder/mlp/mixture_of_experts.py:163-171, 193-196 (routing followed by `get_sparse_map`).
  * `workspace`: fm_sparse_map_from_router_workspace_size(num_tokens, num_experts) bytes, 16-byte aligned. */
@@ -329,30 +334,6 @@ int fm_output_sparse_matmul_gated_activation_backward(const void *lhs, const voi
                                                       int64_t lhs_stride_inner, int64_t rhs_stride_inner,
                                                       int64_t rhs_stride_col, int activation, int dtype,
                                                       int index_dtype, void *stream);
-
-/* ---------------------------------------------------------------------------------------------------------
- * Measurement probes (no counterpart in the reference, not on the MoE path): the ceilings the benchmark sets the
- * kernels' figures against, measured on the device at hand.
- * --------------------------------------------------------------------------------------------------------- */
-
-/* `workgroups` workgroups of 4 wavefronts each issue `iterations` x 32 back-to-back v_mfma_f32_32x32x16_bf16 from
- * registers; operands are zeros (random_operands = 0) or normal(0, sigma) values. `sink` receives 256 floats per
- * workgroup. The work done is fm_probe_mfma_flops(workgroups, iterations). */
-int fm_probe_mfma(void *sink, int64_t workgroups, int64_t iterations, int random_operands, float sigma, void *stream);
-int64_t fm_probe_mfma_flops(int64_t workgroups, int64_t iterations);
-
-/* target[0 .. bytes) = source[0 .. bytes) with 16-byte streaming loads and stores from `workgroups` workgroups of
- * 256 lanes (grid stride). `bytes` a multiple of 16, both pointers 16-byte aligned. */
-int fm_probe_copy(const void *source, void *target, int64_t bytes, int64_t workgroups, void *stream);
-
-/* `workgroups` workgroups (a multiple of 8, one per CU) of 4 wavefronts each stream 64 KiB per iteration from global
- * memory straight into LDS with 16-byte loads, `iterations` times. Workgroups on one XCD form groups of `shared_by`
- * that read the same region of `region_bytes` (a power of two, 64 KiB or more) over and over, so a small region stays in that
- * XCD's L2. A wavefront keeps up to `in_flight` (1 to 3) iterations of 16 loads on their way while it issues the
- * next. `source` holds (workgroups / 8 / shared_by rounded up) * 8 regions; `cycles` receives one int64 per
- * workgroup: the shader clock cycles its loop took. */
-int fm_probe_l2(const void *source, int64_t region_bytes, int64_t shared_by, int64_t workgroups, int64_t iterations,
-                int64_t in_flight, void *cycles, void *stream);
 
 #ifdef __cplusplus
 }

@@ -68,8 +68,8 @@ def test_grouped_gemm_workspace_size_depends_on_the_dimensions_only(library):
     partials = 512 * 256 * 256 * 4  # the pieces of a split last round
     record = 64  # bytes of the tile table per workgroup id
 
-    def ids(row_tiles, column_tiles, split):  # whole rounds of 256 ids, then the pieces
-        return -(-row_tiles * column_tiles // 256) * 256 + (512 if split else 0)
+    def ids(row_tiles, column_tiles, split):  # whole rounds of 256 ids, then the pieces; +4: the table's 64-byte
+        return -(-row_tiles * column_tiles // 256) * 256 + (512 if split else 0) + 4  # header, rounded up to 256 bytes
 
     # Layer 2 forward at the Mixtral shape: 68 + 8 row tiles x 16 column tiles, reduction 14336 -> splits.
     size = library.fm_grouped_gemm_workspace_size(17408, 4096, 14336, 8, 1)
@@ -79,6 +79,11 @@ def test_grouped_gemm_workspace_size_depends_on_the_dimensions_only(library):
     # Layer 1 forward (29 rounds) and a short reduction are not split: the table only.
     assert library.fm_grouped_gemm_workspace_size(17408, 28672, 4096, 8, 1) == ids(76, 112, False) * record
     assert library.fm_grouped_gemm_workspace_size(17408, 4096, 1984, 8, 1) == ids(76, 16, False) * record
+    # Dimensions the matrix-core kernel refuses whatever the strides (reduction not in whole 64-element slices, columns
+    # not in whole 16-byte vectors): the generic kernel takes no workspace.
+    assert library.fm_grouped_gemm_workspace_size(17408, 4096, 1000, 8, 1) == 0
+    assert library.fm_grouped_gemm_workspace_size(17408, 4100, 4096, 8, 1) == 0
+    assert library.fm_input_row_sparse_matmul_workspace_size(14340, 4096, 17408, 8, 1) == 0
     assert library.fm_grouped_gemm_workspace_size(0, 4096, 14336, 8, 1) == 0
     # The row-sparse product never splits: 8 experts x 56 row tiles x 16 column tiles.
     assert library.fm_input_row_sparse_matmul_workspace_size(14336, 4096, 17408, 8, 1) == ids(8 * 56, 16, False) * record

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from fast_llm_amd.functional.config import ActivationType, MLPRecomputeLevel
-from fast_llm_amd.functional.mlp import mlp_autograd, mlp_autograd_looped
+from fast_llm_amd.functional.mlp import mlp_autograd, mlp_autograd_looped, mlp_forward
 from fast_llm_amd.functional.sparse_copy import get_sparse_map
 from fast_llm_amd.layers.moe import DroplessMoEMLP, attach_grad_buffer
 from fast_llm_amd.workloads import WORKLOADS, MoEWorkload, make_inputs
@@ -294,6 +294,38 @@ def test_fused_activation_epilogues_are_bit_identical(activation, recompute_leve
     for name, ours in zip(_NAMES, results[True]):
         assert max_rel_err(ours.cpu(), getattr(expected, name)) <= 1e-2, name
         assert rel_rms_err(ours.cpu(), getattr(expected, name)) <= 1e-2, name
+
+
+def test_activation_fusion_is_chosen_per_call(device):
+    """With the default setting the gated activation rides in layer 1's epilogue exactly where layer 1's output is
+    not stored (full recomputation, inference), and the results equal the unfused ones bit for bit."""
+    from fast_llm_amd import _lib
+    from fast_llm_amd.functional.config import KernelConfig
+
+    assert KernelConfig.fuse_activation is None
+    workload = MoEWorkload("policy", 600, 128, 256, 4, 2, torch.bfloat16)
+    inputs = make_inputs(workload, seed=4)
+    fused_label = "fm_output_sparse_matmul_gated_activation["
+    results = {}
+    for level in MLPRecomputeLevel:
+        with _lib.KernelTimer() as timer:
+            results[level] = _run_dropless(inputs, workload, device, recompute_level=level)
+        labels = set(timer.durations_ms())
+        assert any(label.startswith(fused_label) for label in labels) == (level == MLPRecomputeLevel.full), level
+        assert not any("gated_activation_backward" in label for label in labels)
+    for level in MLPRecomputeLevel:
+        for ours, reference in zip(results[level], results[MLPRecomputeLevel.none]):
+            assert torch.equal(ours, reference)
+    # Inference keeps nothing: fused too, same output.
+    sparse_map = get_sparse_map(inputs.top_experts.to(device), workload.experts)
+    with _lib.KernelTimer() as timer:
+        output, context = mlp_forward(
+            inputs.hidden_states.to(device), inputs.scores.to(device), inputs.weight_1.to(device), None,
+            inputs.weight_2.to(device), None, True, ActivationType.silu, None, False, False, MLPRecomputeLevel.none,
+            True, sparse_map,
+        )  # fmt: skip
+    assert context is None and any(label.startswith(fused_label) for label in timer.durations_ms())
+    assert torch.equal(output, results[MLPRecomputeLevel.none][0])
 
 
 def test_step_replays_from_a_hip_graph(device):

@@ -4,6 +4,7 @@ fast_llm/layers/decoder/mlp/mixture_of_experts.py:243-244) and against autograd 
 import pytest
 import torch
 
+from fast_llm_amd import _lib
 from fast_llm_amd.functional.routing import router, topk_routing
 from oracle import moe_oracle
 
@@ -260,7 +261,9 @@ def test_sparse_map_from_the_routers_counts(tokens, experts, k, shared, zipf, de
         logits += 3 * torch.log(torch.arange(1, experts + 1, dtype=torch.float32) ** -1.2)
     scores, top_experts, _, _, counts = router(logits.to(device), k, shared_experts=shared, return_counts=True)
     total = experts + shared
-    handed = get_sparse_map(top_experts, total, router_counts=counts)
+    with _lib.KernelTimer() as timer:
+        handed = get_sparse_map(top_experts, total, router_counts=counts)
+    assert set(timer.durations_ms()) == {"fm_sparse_map_from_router"}
     counted = get_sparse_map(top_experts, total)
     expected = moe_oracle.sparse_map(top_experts.cpu(), total)
     for name in ("sparse_rows", "expert_ends", "expert_pad_begins"):
@@ -273,6 +276,27 @@ def test_sparse_map_from_the_routers_counts(tokens, experts, k, shared, zipf, de
         get_sparse_map(top_experts[: tokens // 2 + 1], total, router_counts=counts) if tokens > 1 else get_sparse_map(
             top_experts, total + 1, router_counts=counts
         )
+
+
+def test_router_counts_of_edited_selections_are_not_used(device):
+    """Counts belong to the `top_experts` tensor the router returned, as it was: a copy of it, or the tensor itself
+    after an in-place edit (a masking or dropping hook), is counted afresh, and the map is the edited selection's."""
+    from fast_llm_amd.functional.sparse_copy import get_sparse_map
+
+    tokens, experts, k = 3000, 16, 4
+    logits = torch.randn(tokens, experts, generator=torch.Generator().manual_seed(11))
+    _, top_experts, _, _, counts = router(logits.to(device), k, return_counts=True)
+    with _lib.KernelTimer() as timer:
+        copied = get_sparse_map(top_experts.clone(), experts, router_counts=counts)
+    assert set(timer.durations_ms()) == {"fm_sparse_map"}
+    assert torch.equal(copied.sparse_rows, get_sparse_map(top_experts, experts).sparse_rows)
+    top_experts[::3, 0] = (top_experts[::3, 0] + 5) % experts  # the counts no longer describe these selections
+    with _lib.KernelTimer() as timer:
+        edited = get_sparse_map(top_experts, experts, router_counts=counts)
+    assert set(timer.durations_ms()) == {"fm_sparse_map"}
+    expected = moe_oracle.sparse_map(top_experts.cpu(), experts)
+    for name in ("sparse_rows", "expert_ends", "expert_pad_begins"):
+        assert torch.equal(getattr(edited, name).cpu().long(), getattr(expected, name)), name
 
 
 def _rms_norm(hidden: int, device) -> torch.nn.Module:
