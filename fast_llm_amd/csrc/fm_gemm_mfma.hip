@@ -316,6 +316,7 @@ struct TileWork {
 };
 
 constexpr int kXcds = 8, kGroupRows = 8, kChunkTiles = 32;
+constexpr int kHalfTileMaxSlices = 64;  // reductions of this many slices or more have no half tiles (see find_tile)
 
 // Logical order of the tiles of a product whose rows are grouped by expert (output-sparse, input-inner-sparse,
 // dense): expert after expert; within an expert its row tiles (ceil(rows_e / 256)) are cut into ceil(count / 8)
@@ -981,8 +982,15 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         tile.num_slices = (k_last - tile.k_first) / kBK;
         // A tile with at most 128 valid rows (the last row tile of an expert whose padded row count is an odd multiple
         // of 128) is a half tile. The transfers stay as they are (the rows past the valid ones bring zeros or repeats
-        // that nobody reads).
-        tile.half = kFusion == kFusionNone && tile.piece_slot < 0 && work.rows_valid <= kTile / 2;
+        // that nobody reads). Only where the reduction is short: a half tile takes 85 % of a full tile's time, so the
+        // workgroups that got one run ahead of the others of their XCD, and with a long reduction (operand panels of
+        // 2 MiB and more against 4 MiB of L2: the 32 tiles of a chunk share their panels only while they are within
+        // some ten slices of each other) the panels are then fetched again by those that follow. Measured at 64
+        // slices and more: L2-miss traffic 5.6 -> 3.0 and 4.6 -> 3.2 (FETCH_SIZE, layer-1 forward and input gradient of
+        // the Mixtral-like workload) and the launches 2 to 4 % faster with full-cost last tiles; at 12 to 44 slices
+        // the half tiles win by 1.5 to 5 %.
+        tile.half = kFusion == kFusionNone && tile.piece_slot < 0 && work.rows_valid <= kTile / 2 &&
+                    tile.num_slices < kHalfTileMaxSlices;
         return true;
     };
 
