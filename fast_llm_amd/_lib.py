@@ -150,18 +150,22 @@ _active_timer: KernelTimer | None = None
 def call(name: str, device: torch.device, *args, label: str | None = None) -> None:
     """Launch entry point `name` on the current stream of `device` (appended as the last argument) and raise on a
     non-zero status."""
+    if device.index is not None and device.index != torch.cuda.current_device():
+        with torch.cuda.device(device):  # the kernels run on the device that is current
+            return call(name, torch.device("cuda", torch.cuda.current_device()), *args, label=label)
     function = getattr(lib(), name)
-    with torch.cuda.device(device):
-        stream = torch.cuda.current_stream(device)
-        timer = _active_timer
-        if timer is not None:
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record(stream)
+    stream = torch.cuda.current_stream()
+    timer = _active_timer
+    if timer is None:
         status = function(*args, stream.cuda_stream)
-        if timer is not None:
-            end.record(stream)
-            timer.records.append((label or name, start, end))
-    check(status)
+    else:
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        status = function(*args, stream.cuda_stream)
+        end.record(stream)
+        timer.records.append((label or name, start, end))
+    if status != 0:
+        check(status)
 
 
 def require_device(*tensors: torch.Tensor | None) -> torch.device:

@@ -8,8 +8,8 @@
 // (reference semantics: fast_llm/functional/triton/sparse_linear.py:185-258, 310-385, 437-517).
 //
 // Half-precision operands with vectorisable layouts go to the MFMA kernel (fm_gemm_mfma.hip). fp32 operands go to
-// the fp32 matrix-core kernel below (128 x 128 x 16 tiles of v_mfma_f32_32x32x2_f32: true fp32 multiply-adds, which
-// is what the 1e-5 fp32 parity bound needs; 59-63 TFLOP/s at 16384 x 4096 x 2048 over 8 experts). Everything else
+// the fp32 matrix-core kernel below (tiles of v_mfma_f32_32x32x2_f32: true fp32 multiply-adds, which is what the
+// 1e-5 fp32 parity bound needs; 59-63 TFLOP/s at 16384 x 4096 x 2048 over 8 experts). Everything else
 // (half-precision operands with odd strides or sizes) goes to the generic kernel: a 64 x 64 x 16 LDS-tiled kernel of
 // scalar multiply-adds. Both compute a row block that straddles an expert boundary in one pass per expert, so they
 // take any padding multiple, and both check every bound.
@@ -168,28 +168,36 @@ __global__ __launch_bounds__(kGenThreads) void grouped_gemm_generic_kernel(GemmA
 // =========================================================================================================
 // fp32 operands on the matrix cores
 // =========================================================================================================
-// 128 x 128 output tile per workgroup, 4 wavefronts (2 x 2), each 64 x 64 as 2 x 2 accumulators of
-// v_mfma_f32_32x32x2_f32 (true fp32 multiply-adds: the 1e-5 parity bound holds), K in slices of 16. Operands of any
+// kTile x kTile output tile per workgroup, 4 wavefronts (2 x 2), each kTile / 2 squared as accumulators of
+// v_mfma_f32_32x32x2_f32 (true fp32 multiply-adds: the 1e-5 parity bound holds), K in slices of kK. Operands of any
 // strides are fetched element by element (consecutive lanes along the axis with the smaller stride) into registers
 // one slice ahead and stored to LDS as [k][row], double-buffered, one barrier per slice; several workgroups share a
-// CU. Tiles lie on a fixed 128-row grid: one that straddles an expert boundary is computed in one pass per expert,
-// like the generic kernel's, so any padding multiple works (the reference's multiple of 128 gives one pass).
+// CU. Tiles lie on a fixed grid of kTile rows: one that straddles an expert boundary is computed in one pass per
+// expert, like the generic kernel's, so any padding multiple works (the reference's multiple of 128 gives one pass).
+// Two shapes: 128 x 128 x 16 for launches that fill the device (59-63 TFLOP/s at 16384 x 4096 x 2048 over 8 experts),
+// and 64 x 64 x 32 for launches of fewer 128-tiles than there are CUs (the 512-token configuration: 32 to 128 of
+// them), which are bound by the memory latency of one slice after the other: four times the workgroups, each with a
+// quarter of the multiply-adds and half the slices.
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float gemm_f32x16_t;
-constexpr int kF32Tile = 128, kF32K = 16, kF32Threads = 256;
-constexpr int kF32Pitch = kF32Tile + 4;                               // floats per K-row in LDS; +4 spreads the banks
-constexpr int kF32PerThread = kF32Tile * kF32K / kF32Threads;         // operand elements per thread and slice: 8
+constexpr int kF32Tile = 128, kF32SmallTile = 64, kF32Threads = 256;
+constexpr int kF32SmallLaunchTiles = 256;  // fewer 128-tiles than this (the CUs of the device): tiles of 64
 
+template <int kTile, int kK>
 __global__ __launch_bounds__(kF32Threads) void grouped_gemm_f32_mfma_kernel(GemmArgs args) {
-    __shared__ float lds_a[2][kF32K][kF32Pitch];
-    __shared__ float lds_b[2][kF32K][kF32Pitch];
+    constexpr int kPitch = kTile + 4;                       // floats per K-row in LDS; +4 spreads the banks
+    constexpr int kPerThread = kTile * kK / kF32Threads;    // operand elements per thread and slice
+    constexpr int kWaveTile = kTile / 2, kBlocks = kWaveTile / 32;  // a wavefront's part, in 32 x 32 accumulators
+    static_assert(kPerThread * kF32Threads == kTile * kK && kBlocks >= 1 && kK % 2 == 0, "tile shape");
+    __shared__ float lds_a[2][kK][kPitch];
+    __shared__ float lds_b[2][kK][kPitch];
     const int tile_n = blockIdx.x % args.tiles_n, tile_m = blockIdx.x / args.tiles_n;
-    const int64_t row0 = static_cast<int64_t>(tile_m) * kF32Tile, col0 = static_cast<int64_t>(tile_n) * kF32Tile;
+    const int64_t row0 = static_cast<int64_t>(tile_m) * kTile, col0 = static_cast<int64_t>(tile_n) * kTile;
     int64_t rows_here = args.rows - row0, cols_here = args.cols - col0;
     if (args.mode == kInputRowSparse) {
         const int64_t left_in_expert = args.sparse_size - row0 % args.sparse_size;
         if (left_in_expert < rows_here) rows_here = left_in_expert;
     }
-    if (rows_here > kF32Tile) rows_here = kF32Tile;
+    if (rows_here > kTile) rows_here = kTile;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wave_m = wave >> 1, wave_n = wave & 1;
     const bool lhs_k_fastest = args.lhs_stride_inner <= args.lhs_stride_row;
@@ -197,32 +205,32 @@ __global__ __launch_bounds__(kF32Threads) void grouped_gemm_f32_mfma_kernel(Gemm
     const float *lhs_all = static_cast<const float *>(args.lhs), *rhs_all = static_cast<const float *>(args.rhs);
 
     for (int first_row = 0; first_row < rows_here;) {
-        const TileWork work = resolve_tile(args, row0, col0, first_row, kF32Tile);
+        const TileWork work = resolve_tile(args, row0, col0, first_row, kTile);
         if (work.skip) return;  // the rest of the tile lies past the last expert
         const int row_hi = work.row_hi < rows_here ? work.row_hi : static_cast<int>(rows_here);
         const float *lhs = lhs_all + work.lhs_offset, *rhs = rhs_all + work.rhs_offset;
-        gemm_f32x16_t acc[2][2];
+        gemm_f32x16_t acc[kBlocks][kBlocks];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < kBlocks; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < kBlocks; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
         // Element e of this thread in a slice: (k, row) with the memory-contiguous axis fastest over the lanes.
-        float staged_a[kF32PerThread], staged_b[kF32PerThread];
+        float staged_a[kPerThread], staged_b[kPerThread];
         auto fetch = [&](int64_t k0) {
 #pragma unroll
-            for (int e = 0; e < kF32PerThread; ++e) {
+            for (int e = 0; e < kPerThread; ++e) {
                 const int i = threadIdx.x + e * kF32Threads;
-                int k_local = lhs_k_fastest ? i % kF32K : i / kF32Tile;
-                const int r_local = lhs_k_fastest ? i / kF32K : i % kF32Tile;
+                int k_local = lhs_k_fastest ? i % kK : i / kTile;
+                const int r_local = lhs_k_fastest ? i / kK : i % kTile;
                 int64_t k = k0 + k_local;
                 staged_a[e] = 0.f;
                 if (r_local >= first_row && r_local < row_hi && k >= work.k_lo && k < work.k_hi)
                     staged_a[e] = lhs[r_local * args.lhs_stride_row + k * args.lhs_stride_inner];
-                k_local = rhs_k_fastest ? i % kF32K : i / kF32Tile;
-                const int c_local = rhs_k_fastest ? i / kF32K : i % kF32Tile;
+                k_local = rhs_k_fastest ? i % kK : i / kTile;
+                const int c_local = rhs_k_fastest ? i / kK : i % kTile;
                 k = k0 + k_local;
                 staged_b[e] = 0.f;
                 if (c_local < cols_here && k >= work.k_lo && k < work.k_hi)
@@ -231,36 +239,36 @@ __global__ __launch_bounds__(kF32Threads) void grouped_gemm_f32_mfma_kernel(Gemm
         };
         auto stage = [&](int buffer) {
 #pragma unroll
-            for (int e = 0; e < kF32PerThread; ++e) {
+            for (int e = 0; e < kPerThread; ++e) {
                 const int i = threadIdx.x + e * kF32Threads;
-                lds_a[buffer][lhs_k_fastest ? i % kF32K : i / kF32Tile][lhs_k_fastest ? i / kF32K : i % kF32Tile] = staged_a[e];
-                lds_b[buffer][rhs_k_fastest ? i % kF32K : i / kF32Tile][rhs_k_fastest ? i / kF32K : i % kF32Tile] = staged_b[e];
+                lds_a[buffer][lhs_k_fastest ? i % kK : i / kTile][lhs_k_fastest ? i / kK : i % kTile] = staged_a[e];
+                lds_b[buffer][rhs_k_fastest ? i % kK : i / kTile][rhs_k_fastest ? i / kK : i % kTile] = staged_b[e];
             }
         };
 
-        const int64_t k_begin = work.k_lo / kF32K * kF32K;
+        const int64_t k_begin = work.k_lo / kK * kK;
         if (k_begin < work.k_hi) {
             fetch(k_begin);
             stage(0);
         }
         __syncthreads();
         int buffer = 0;
-        for (int64_t k0 = k_begin; k0 < work.k_hi; k0 += kF32K, buffer ^= 1) {
-            const bool more = k0 + kF32K < work.k_hi;
-            if (more) fetch(k0 + kF32K);  // in flight during the multiplications
+        for (int64_t k0 = k_begin; k0 < work.k_hi; k0 += kK, buffer ^= 1) {
+            const bool more = k0 + kK < work.k_hi;
+            if (more) fetch(k0 + kK);  // in flight during the multiplications
 #pragma unroll
-            for (int kstep = 0; kstep < kF32K / 2; ++kstep) {
+            for (int kstep = 0; kstep < kK / 2; ++kstep) {
                 // Lane l supplies row (or column) l % 32 at k = 2 kstep + l / 32.
                 const int k_local = 2 * kstep + (lane >> 5);
-                float a[2], b[2];
+                float a[kBlocks], b[kBlocks];
 #pragma unroll
-                for (int i = 0; i < 2; ++i) a[i] = lds_a[buffer][k_local][wave_m * 64 + i * 32 + (lane & 31)];
+                for (int i = 0; i < kBlocks; ++i) a[i] = lds_a[buffer][k_local][wave_m * kWaveTile + i * 32 + (lane & 31)];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) b[j] = lds_b[buffer][k_local][wave_n * 64 + j * 32 + (lane & 31)];
+                for (int j = 0; j < kBlocks; ++j) b[j] = lds_b[buffer][k_local][wave_n * kWaveTile + j * 32 + (lane & 31)];
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < kBlocks; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
+                    for (int j = 0; j < kBlocks; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
             }
             // The other buffer was last read a slice ago, before the previous barrier.
@@ -270,14 +278,14 @@ __global__ __launch_bounds__(kF32Threads) void grouped_gemm_f32_mfma_kernel(Gemm
 
         // Lane l holds column l % 32 of each 32 x 32 accumulator; register v is row 8 (v / 4) + 4 (l / 32) + v % 4.
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < kBlocks; ++i)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = wave_m * 64 + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + v % 4;
+                const int row = wave_m * kWaveTile + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + v % 4;
                 if (row < first_row || row >= row_hi) continue;
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int column = wave_n * 64 + j * 32 + (lane & 31);
+                for (int j = 0; j < kBlocks; ++j) {
+                    const int column = wave_n * kWaveTile + j * 32 + (lane & 31);
                     if (column >= cols_here) continue;
                     store_out_dyn(args.out, args.out_dtype,
                                   work.out_offset + row * args.out_stride_row + column * args.out_stride_col,
@@ -314,16 +322,23 @@ static int run_gemm(const char *name, GemmArgs args, int dtype, void *workspace,
         if (args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % kGenTile != 0)
             return fail(FM_ERR_UNSUPPORTED, "%s: row_sparse_dim=%lld must be a multiple of %d", name,
                         (long long)args.sparse_size, kGenTile);
-        // fp32 operands go to the matrix cores when the row-sparse product's blocks of out are whole tiles there too.
-        const bool f32_mfma = dtype == FM_DTYPE_F32 &&
-                              !(args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % kF32Tile != 0);
-        const int tile = f32_mfma ? kF32Tile : kGenTile;
+        // fp32 operands go to the matrix cores when the row-sparse product's blocks of out are whole tiles there too:
+        // tiles of 128, or of 64 when there are fewer 128-tiles than CUs (see the kernel).
+        const auto whole_tiles = [&](int tile) {
+            return !(args.mode == kInputRowSparse && args.num_experts > 1 && args.sparse_size % tile != 0);
+        };
+        const int64_t large_tiles = ((args.rows + kF32Tile - 1) / kF32Tile) * ((args.cols + kF32Tile - 1) / kF32Tile);
+        const bool f32_small = dtype == FM_DTYPE_F32 && large_tiles < kF32SmallLaunchTiles && whole_tiles(kF32SmallTile);
+        const bool f32_mfma = dtype == FM_DTYPE_F32 && (f32_small || whole_tiles(kF32Tile));
+        const int tile = f32_small ? kF32SmallTile : (f32_mfma ? kF32Tile : kGenTile);
         args.tiles_m = static_cast<int>((args.rows + tile - 1) / tile);
         args.tiles_n = static_cast<int>((args.cols + tile - 1) / tile);
         FM_REQUIRE(static_cast<int64_t>(args.tiles_m) * args.tiles_n < (int64_t(1) << 31), "%s: too many tiles", name);
         const int grid = args.tiles_m * args.tiles_n;
-        if (f32_mfma) {
-            grouped_gemm_f32_mfma_kernel<<<grid, kF32Threads, 0, stream>>>(args);
+        if (f32_small) {
+            grouped_gemm_f32_mfma_kernel<kF32SmallTile, 32><<<grid, kF32Threads, 0, stream>>>(args);
+        } else if (f32_mfma) {
+            grouped_gemm_f32_mfma_kernel<kF32Tile, 16><<<grid, kF32Threads, 0, stream>>>(args);
         } else {
             FM_DISPATCH_DTYPE(dtype, T, { grouped_gemm_generic_kernel<T><<<grid, kGenThreads, 0, stream>>>(args); });
         }

@@ -307,10 +307,13 @@ def test_mfma_kernel_on_ragged_experts(experts, dense_dim, sparse_dim, dtype, de
 # The matrix-core kernel counts by hand which of its transfers have landed when a K-step reads them, with one count
 # per load schedule (K-contiguous rhs, row-contiguous rhs, weight gradient) and tile kind (whole, half: an expert's last
 # row tile with at most 128 valid rows). Every number of 64-wide reduction slices from 1 to 10 through all of them:
-# experts of 256 + 128 rows (a whole and a half tile), of 128 rows (a half tile) and of 512 rows; the walk of a
-# workgroup over several tiles comes with the 40 column tiles of the second size.
+# experts of 256 + 128 rows (a whole and a half tile), of 128 rows (a half tile) and of 512 rows; one column tile, five
+# whole ones followed by one of 72 columns, and the walk of a workgroup over several tiles with 40 column tiles.
 @pytest.mark.parametrize(
-    ("slices", "other"), [(slices, 256) for slices in range(1, 11)] + [(slices, 40 * 256) for slices in (1, 2, 3, 6, 9)]
+    ("slices", "other"),
+    [(slices, 256) for slices in range(1, 11)]
+    + [(slices, 5 * 256 + 72) for slices in range(1, 11)]
+    + [(slices, 40 * 256) for slices in (1, 2, 3, 6, 9)],
 )
 def test_every_slice_count_through_the_pipeline(slices, other, device):
     dtype = torch.bfloat16
