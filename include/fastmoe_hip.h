@@ -8,7 +8,8 @@
  *     returns: outputs and every workspace are the caller's, and a workspace may be reused as soon as the stream
  *     has passed the call;
  *   - returns `FM_OK` (0), a positive remark (the work was launched), or a negative `fm_status`; the message of a
- *     negative status for the calling thread is read with `fm_last_error()`. No C++ exception crosses this boundary.
+ *     negative status for the calling thread is read with `fm_last_error()`. Only negative values are errors: test
+ *     `status < 0`, not `status != FM_OK` (a remark leaves no message). No C++ exception crosses this boundary.
  *
  * The reference (ServiceNow/Fast-LLM) has no FFI for this path: its "operator API" is a set of Python
  * callables that launch Triton kernels. Each function below replaces the kernel launch inside one of those
