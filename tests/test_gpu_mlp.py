@@ -40,7 +40,7 @@ _NAMES = ("output", "grad_input", "grad_scores", "grad_weight_1", "grad_weight_2
 
 def test_dropless_mlp_like_the_reference(device):
     """tests/functional/test_functional.py:89-183: dropless vs looped within the reference's rms thresholds, and
-    bit-equal results for all four recompute levels."""
+    bit-equal results for all four recompute levels; both also against the CPU oracle."""
     fixture = REFERENCE_FIXTURES["dropless_mlp"]
     experts, top_k, std = fixture["experts"], fixture["experts_per_token"], fixture["std"]
     tokens, hidden, ffn = fixture["tokens"], fixture["hidden"], fixture["ffn"]
@@ -87,6 +87,15 @@ def test_dropless_mlp_like_the_reference(device):
             # fp32 here, so the tighter benchmark bound holds as well
             assert max_rel_err(output, output_ref) <= 1e-5
             assert max_rel_err(input_.grad, input_grad_ref) <= 1e-5
+            # The looped path above runs on this library's own kernels too; the CPU oracle's looped MoE is the
+            # independent check of both.
+            expected = moe_oracle.looped_moe_forward_backward(
+                input_.detach().cpu(), scores.detach().cpu(), top_experts.cpu(), weight_1.detach().cpu(),
+                weight_2.detach().cpu(), experts, output_grad.cpu(),
+            )  # fmt: skip
+            ours = (output, input_.grad, scores.grad, weight_1.grad_buffer, weight_2.grad_buffer)
+            for name, tensor in zip(_NAMES, ours):
+                assert max_rel_err(tensor.detach().cpu(), getattr(expected, name)) <= 1e-5, name
             output_ref, input_grad_ref, scores_grad_ref = output, input_.grad, scores.grad
             param_grad_refs = [param.grad_buffer for param in params]
         else:
