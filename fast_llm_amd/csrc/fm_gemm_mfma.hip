@@ -468,7 +468,12 @@ __device__ __forceinline__ int logical_of_block(int pid) {
     // often half tiles and shorter, would otherwise always fall to the same CUs, and those would run further and
     // further ahead of the CUs they share operand panels with.
     const int round = local / kChunkTiles;
-    return (round * kXcds + xcd) * kChunkTiles + (local + round * kSlotRotation) % kChunkTiles;
+    // Which of the round's eight chunks an XCD takes rotates as well. With chunk c always on XCD c % 8 the XCDs ran
+    // the products whose rows are grouped by expert at paces that differed by up to +-5 % launch after launch (the same
+    // XCDs always ahead, the weight-gradient product within +-0.4 %): chunks of one residue are not the same work as
+    // chunks of another (they meet the expert and row-group boundaries at different places). Rotated, every XCD sees
+    // every residue (Mixtral-like step -0.9 %, measured A-B-A-B; what is left of the spread is the XCDs' own).
+    return (round * kXcds + (xcd + round) % kXcds) * kChunkTiles + (local + round * kSlotRotation) % kChunkTiles;
 }
 
 // ---- splitting the reduction of the last tiles ---------------------------------------------------------------
