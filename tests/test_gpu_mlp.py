@@ -196,12 +196,20 @@ def test_moe_module_routes_and_runs(device):
         assert torch.equal(layer(x), out)
 
 
-@pytest.mark.parametrize("name", ["mixtral", "fine_grained", "wide", "imbalanced", "imbalanced_empty"])
+@pytest.mark.parametrize(
+    "name", ["mixtral", "fine_grained", "wide", "imbalanced", "imbalanced_empty", "beyond_int32_elements"]
+)
 def test_benchmark_configurations_full_size(name, device):
     """Configurations 2-5 at full size. The CPU oracle would need minutes per case, so the checker is the oracle's
-    looped MoE evaluated by torch on the GPU in fp32 (per-expert dense matmuls + autograd) on the same inputs."""
+    looped MoE evaluated by torch on the GPU in fp32 (per-expert dense matmuls + autograd) on the same inputs.
+    The last case is a size no benchmark has: 69 001 tokens to 8 of 16 experts, i.e. 552 008 sparse rows of 4096, so that
+    the dispatched rows, the layer-1 output and the layer-2 output each hold more than 2^31 elements (4.5 GB):
+    element offsets that do not fit 32 bits in every kernel of the path."""
     if name == "imbalanced_empty":
         workload = MoEWorkload(name, 8192, 4096, 14336, 8, 2, torch.bfloat16, zipf_exponent=1.2, empty_experts=(5,))
+    elif name == "beyond_int32_elements":
+        workload = MoEWorkload(name, 69001, 4096, 2048, 16, 8, torch.bfloat16)
+        assert workload.sparse_rows_unpadded * workload.hidden > 2**31
     else:
         workload = WORKLOADS[name]
     inputs = make_inputs(workload, seed=7)

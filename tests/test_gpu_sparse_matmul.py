@@ -593,3 +593,46 @@ def test_half_precision_on_the_generic_kernel_warns(device):
         warnings.simplefilter("error")
         dense_matmul(_normal(128, 128, torch.bfloat16, generator).to(device), _normal(128, 72, torch.bfloat16, generator).to(device))
         dense_matmul(lhs.float().to(device), rhs.float().to(device))  # fp32 belongs on that kernel: no remark
+
+
+def test_one_expert_of_more_than_4_gib(device):
+    """An expert whose rows span more than 4 GiB of a row-major operand (528 384 rows of 4096 bf16 values = 4.33 GB,
+    after a first expert of 256 rows): byte offsets inside one expert's block exceed 32 bits in all three products,
+    along the rows of the output-sparse and inner-sparse products and along the reduction of the row-sparse one
+    (8256 slices of 64). Operands are drawn on the GPU and the checker is the oracle evaluated there in fp32: on the CPU
+    it would take minutes."""
+    dtype, wide, narrow = torch.bfloat16, 4096, 256
+    case = {"expert_ends": [256, 256 + 528384], "tokens_per_expert": [200, 528300]}
+    oracle_map = fixture_sparse_map(case)
+    sparse_map = to_device_map(oracle_map, device)
+    rows = oracle_map.num_rows
+    assert (rows - 256) * wide * dtype.itemsize > 2**32
+    generator = torch.Generator(device=device).manual_seed(5)
+
+    def normal(*shape):
+        return torch.empty(shape, dtype=dtype, device=device).normal_(0, _STD, generator=generator)
+
+    x, y = normal(rows, wide), normal(rows, narrow)
+    weight = normal(2 * narrow, wide)
+    # Output-sparse: [rows, 4096] x [4096, 2 * 256] -> [rows, 256]; the lhs block of the second expert is the large one.
+    out = output_sparse_matmul(x, weight.t(), sparse_map)
+    expected = moe_oracle.output_sparse_matmul(x.float(), weight.t().float(), oracle_map)
+    assert max_rel_err(out, expected) <= _MAX_REL[dtype]
+    # Inner-sparse: [rows, 256] x [2 * 256, 4096] -> [rows, 4096]; the output block of the second expert.
+    out = input_inner_sparse_matmul(y, weight, sparse_map)
+    expected = moe_oracle.input_inner_sparse_matmul(y.float(), weight.float(), oracle_map)
+    assert max_rel_err(out, expected) <= _MAX_REL[dtype]
+    assert max_rel_err(out[-512:], expected[-512:]) <= _MAX_REL[dtype]
+    del out, expected
+    # Row-sparse: [256, rows] x [rows, 4096] -> [2 * 256, 4096]; the reduction runs down the large block, padding
+    # rows (poisoned) excluded.
+    real = oracle_map.real_row_mask().to(device)
+    x[~real] = float("nan")
+    y[~real] = float("nan")
+    out = input_row_sparse_matmul(y.t(), x, sparse_map)
+    x[~real] = 0
+    y[~real] = 0
+    expected = moe_oracle.input_row_sparse_matmul(y.t().float(), x.float(), oracle_map)
+    assert torch.isfinite(out).all()
+    assert max_rel_err(out, expected) <= _MAX_REL[dtype]
+    assert max_rel_err(out[:narrow], expected[:narrow]) <= _MAX_REL[dtype]
