@@ -23,6 +23,7 @@ file, built into `libbench_probes.so` by `build_probes()` (which `__graft_entry_
 """
 
 import argparse
+import contextlib
 import ctypes
 import json
 import os
@@ -189,8 +190,12 @@ def cpu_baseline(workload, inputs, tokens: int, repetitions: int = 3) -> dict:
     }
 
 
-def time_workload(workload, args, steps: int, warmup: int, grad_dtype_name: str, recompute_level, device) -> dict:
-    """Warm up, time `steps` steps of `workload` and return the step time and the per-kernel figures."""
+def time_workload(
+    workload, args, steps: int, warmup: int, grad_dtype_name: str, recompute_level, device, events: bool = True
+) -> dict:
+    """Warm up, time `steps` steps of `workload` and return the step time and the per-kernel figures. Without `events`
+    the timed steps carry no HIP events at all (for a step that is bound by the host's launches) and every kernel
+    figure comes from the pass that follows them."""
     from fast_llm_amd import _lib
     from fast_llm_amd.functional.config import ActivationType
     from fast_llm_amd.functional.mlp import mlp_autograd
@@ -218,15 +223,28 @@ def time_workload(workload, args, steps: int, warmup: int, grad_dtype_name: str,
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    with _lib.KernelTimer() as timer:
+    # The timed region. HIP events bracket the grouped products only (the kernel the roofline figure is about): every
+    # event record is a marker that the next kernel waits behind, and bracketing all ~22 calls of a step costs 0.06-0.1
+    # ms per step (0.6 % of the Mixtral-like step, 1.6 % of the wide one, a third of the 512-token one).
+    timer = _lib.KernelTimer(only="matmul") if events else None
+    with timer or contextlib.nullcontext():
         start = time.perf_counter()
         for _ in range(steps):
             step()
         torch.cuda.synchronize()
         seconds = time.perf_counter() - start
     ms_per_step = seconds / steps * 1e3
-    all_durations = timer.durations_ms()
+    all_durations = timer.durations_ms() if timer else {}
     calls_per_step = {label: len(values) / steps for label, values in all_durations.items()}
+    # The other kernels of the step: a second, shorter pass with events around every call.
+    other_steps = min(steps, 10)
+    with _lib.KernelTimer() as timer:
+        for _ in range(other_steps):
+            step()
+    for label, values in timer.durations_ms().items():
+        if label not in all_durations:
+            all_durations[label] = values
+            calls_per_step[label] = len(values) / other_steps
     kernels = {
         label: kernel_figures(label, values, workload, recompute_level) | {"calls_per_step": calls_per_step[label]}
         for label, values in sorted(all_durations.items())
@@ -665,8 +683,10 @@ def main() -> None:
             if name == workload.name:
                 continue
             other_workload = WORKLOADS[name]
-            config_timed = time_workload(other_workload, args, min(args.steps, 10), min(args.warmup, 2), "same",
-                                         recompute_level, device)  # fmt: skip
+            # A few steps each; the 512-token one is bound by the host's launches and needs more to be steady.
+            config_steps, config_warmup = (200, 20) if name == "tiny" else (min(args.steps, 10), min(args.warmup, 2))
+            config_timed = time_workload(other_workload, args, config_steps, config_warmup, "same",
+                                         recompute_level, device, events=name != "tiny")  # fmt: skip
             configs[name] = summary_of(other_workload, config_timed)
             if name != "imbalanced":  # same shapes as the Mixtral-like configuration
                 isolated = isolated_kernels(other_workload, config_timed["inputs"], device, recompute_level)
