@@ -966,18 +966,9 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         int num_slices;
         bool half;        // at most 128 valid rows: the wavefronts share them, 64 each, and issue half the MFMAs
     };
-    auto find_tile = [&](int id, Tile &tile) -> bool {
-        if (args.tile_table != nullptr) {
-            // One scalar load (the table was written by an earlier kernel, so the scalar cache cannot hold stale lines).
-            typedef __attribute__((__vector_size__(16 * sizeof(uint32_t)))) uint32_t u32x16_t;
-            const TileRecord *address = static_cast<const TileRecord *>(args.tile_table) + id;
-            u32x16_t raw;
-            asm volatile("s_load_dwordx16 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(raw) : "s"(address) : "memory");
-            tile.work = __builtin_bit_cast(TileRecord, raw);
-            if (!tile.work.found) return false;
-        } else if (!compute_tile_record(args, id, tile.work)) {
-            return false;
-        }
+    typedef __attribute__((__vector_size__(16 * sizeof(uint32_t)))) uint32_t u32x16_t;
+    // The rest of `tile` from its record.
+    auto finish_tile = [&](Tile &tile) {
         const TileRecord &work = tile.work;
         tile.piece_slot = work.piece_slot;
         // Slices start at multiples of kBK, except where both operands are row-contiguous (any K-row can start a
@@ -996,6 +987,53 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         // the half tiles win by 1.5 to 5 %.
         tile.half = kFusion == kFusionNone && tile.piece_slot < 0 && work.rows_valid <= kTile / 2 &&
                     tile.num_slices < kHalfTileMaxSlices;
+    };
+    auto find_tile = [&](int id, Tile &tile) -> bool {
+        if (args.tile_table != nullptr) {
+            // One scalar load (the table was written by an earlier kernel, so the scalar cache cannot hold stale lines).
+            const TileRecord *address = static_cast<const TileRecord *>(args.tile_table) + id;
+            u32x16_t raw;
+            asm volatile("s_load_dwordx16 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(raw) : "s"(address) : "memory");
+            tile.work = __builtin_bit_cast(TileRecord, raw);
+            if (!tile.work.found) return false;
+        } else if (!compute_tile_record(args, id, tile.work)) {
+            return false;
+        }
+        finish_tile(tile);
+        return true;
+    };
+    // The record of the tile AFTER the next one is requested a whole tile ahead, so that nobody waits for it (the
+    // scalar load above takes 0.6 us, of tiles that take 17 to 50 us where the reduction is short): a load straight
+    // into LDS, issued right after the next tile's first loads, i.e. before the current tile is written out. It lands
+    // in the last 256 bytes of the middle lhs slot, which the epilogue's staging area does not reach and which the
+    // next tile's loads fill only in their third K-step; lane l fetches word l % 16 of the record, every wavefront
+    // fetches it for itself (the same bytes to the same place) and reads it back once its own loads up to that one
+    // have landed, before the barrier that starts the tile. The words then wait in one register per lane.
+    constexpr int kRecordSpot = kLdsBytes - kOperandBytes - 256;
+    static_assert(kStagingBase + kWaves * 32 * (kWaveCols * 4 + kEpiloguePadBytes) <= kRecordSpot, "record spot is staging");
+    auto request_record = [&](int id) {
+        const TileRecord *address = static_cast<const TileRecord *>(args.tile_table) + id;
+        const __amdgpu_buffer_rsrc_t resource = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char *>(uniform_pointer(reinterpret_cast<const char *>(address))), 0,
+            static_cast<int>(sizeof(TileRecord)), kBufferResourceFlags);
+        const uint32_t lane_offset = (opaque(static_cast<int>(threadIdx.x)) & 15) * 4;
+        const int spot = __builtin_amdgcn_readfirstlane(kRecordSpot);
+        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds"
+                     :
+                     : "s"(spot), "v"(lane_offset), "s"(resource)
+                     : "memory");
+    };
+    auto read_record = [&]() -> uint32_t {
+        const int lane_offset = (opaque(static_cast<int>(threadIdx.x)) & 15) * 4;
+        return *reinterpret_cast<FM_LDS(const uint32_t) *>(lds + kRecordSpot + lane_offset);
+    };
+    auto tile_of_record = [&](uint32_t words, Tile &tile) -> bool {
+        u32x16_t raw;
+#pragma unroll
+        for (int word = 0; word < 16; ++word) raw[word] = __builtin_amdgcn_readlane(words, word);
+        tile.work = __builtin_bit_cast(TileRecord, raw);
+        if (!tile.work.found) return false;
+        finish_tile(tile);
         return true;
     };
 
@@ -1222,14 +1260,23 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
     constexpr int kLoadsAfterSlice0 = kLoadsPerOperand + kPrologueRhs + kPrologueLhs;
 
     first_loads(tile);
+    // Whether the record of the id after `id` has been requested (with a tile table, for every id that exists).
+    bool requested = false;
+    auto request_next_record = [&]() {
+        requested = args.tile_table != nullptr && id + static_cast<int>(gridDim.x) < args.num_ids;
+        if (requested) request_record(id + gridDim.x);
+    };
+    request_next_record();
     while (true) {
         setup_tile(tile);
         const int num_slices = tile.num_slices;
+        uint32_t next_record = 0;
         if (num_slices > 0) {
             // Prologue: slice 0, lhs slice 1 and the first pieces of the slices after them on their way; slice 0 landed.
             continue_tile();
             clear_accumulators();  // 256 register writes, while the first loads are on their way
-            wait_for_loads<kLoadsAfterSlice0>();  // slice 0 was loaded first
+            wait_for_loads<kLoadsAfterSlice0>();  // slice 0 was loaded first, the next record right after it
+            if (requested) next_record = read_record();
             __syncthreads();
             mask_slice(0, lhs_now, 0);
 #pragma unroll
@@ -1256,6 +1303,10 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
             wait_for_loads<0>();  // the zero-filling loads of slices past the end still write LDS
         } else {
             clear_accumulators();
+            if (requested) {
+                wait_for_loads<0>();
+                next_record = read_record();
+            }
         }
         __syncthreads();  // all wavefronts are done reading operand slices; LDS becomes the staging area
         forget_arguments();
@@ -1268,8 +1319,11 @@ __global__ __launch_bounds__(kMfmaThreads, kWaves / 4) void grouped_gemm_mfma_ke
         // The next tile is looked up here, not earlier, to keep its coordinates out of the registers of the main loop;
         // its first loads go out before this tile's results do.
         id += gridDim.x;
-        const bool have_next = id < args.num_ids && find_tile(id, tile);
-        if (have_next) first_loads(tile);
+        const bool have_next = requested ? tile_of_record(next_record, tile) : id < args.num_ids && find_tile(id, tile);
+        if (have_next) {
+            first_loads(tile);
+            request_next_record();
+        }
 
         FM_LDS(char) *staging = lds + kStagingBase;
         const int lane = opaque(static_cast<int>(threadIdx.x & 63));  // per-lane addresses of the epilogue: not hoisted
