@@ -269,10 +269,14 @@ __device__ __forceinline__ int fragment_base(int row_base, int q, int lane) {
 // `bases`: fragment_base of q = 0..3 plus the LDS offset of the operand's slot 0.
 template <bool kContiguousK>
 __device__ __forceinline__ u32x4_t load_fragment(FM_LDS(char) * lds, const int (&bases)[4], int slot, int i, int kstep) {
+    // The kernel's only LDS is the dynamic allocation, which starts at LDS address 0 (the transfers above put absolute
+    // addresses into M0 as well). The address of that array is not a constant the compiler knows, though: formed as
+    // `lds + offset`, every fragment address costs an addition of zero in the main loop.
+    (void)lds;
     if constexpr (kContiguousK) {
-        return *reinterpret_cast<FM_LDS(u32x4_t) *>(lds + bases[kstep] + (slot * kOperandBytes + i * 32 * kBK * 2));
+        return *(FM_LDS(u32x4_t) *)static_cast<uint32_t>(bases[kstep] + (slot * kOperandBytes + i * 32 * kBK * 2));
     } else {
-        FM_LDS(char) *address = lds + bases[i] + (slot * kOperandBytes + kstep * 16 * kTile * 2);
+        FM_LDS(char) *address = (FM_LDS(char) *)static_cast<uint32_t>(bases[i] + (slot * kOperandBytes + kstep * 16 * kTile * 2));
         const i16x4_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<FM_LDS(i16x4_t) *>(address));
         const i16x4_t high =
             __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<FM_LDS(i16x4_t) *>(address + 4 * kTile * 2));
