@@ -636,3 +636,48 @@ def test_one_expert_of_more_than_4_gib(device):
     assert torch.isfinite(out).all()
     assert max_rel_err(out, expected) <= _MAX_REL[dtype]
     assert max_rel_err(out[:narrow], expected[:narrow]) <= _MAX_REL[dtype]
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_launches_of_many_rounds(block, device):
+    """Random ragged layouts large enough for launches of several rounds of workgroups (hundreds to thousands of tiles:
+    the tile table, a workgroup walking from tile to tile, half tiles, experts without tokens, split last rounds),
+    all three products. Operands are drawn on the GPU and the checker is the oracle evaluated there in fp32."""
+    for seed in range(30 * block, 30 * (block + 1)):
+        generator = torch.Generator().manual_seed(5000 + seed)
+
+        def pick(*choices):
+            return choices[int(torch.randint(0, len(choices), (1,), generator=generator))]
+
+        experts = pick(2, 5, 8, 16, 40)
+        inner = pick(64, 192, 448, 768, 1408, 2048, 4096)
+        other = pick(256, 520, 1024, 1408, 2112)
+        dtype = pick(torch.bfloat16, torch.float16)
+        tokens = torch.randint(0, pick(300, 900, 2500), (experts,), generator=generator)
+        if pick(True, False):
+            tokens[int(torch.randint(0, experts, (1,), generator=generator))] = 0
+        ends = torch.cumsum((tokens + 127) // 128 * 128, 0)
+        if int(ends[-1]) == 0:
+            continue
+        oracle_map = fixture_sparse_map({"expert_ends": ends.tolist(), "tokens_per_expert": tokens.tolist()})
+        sparse_map = to_device_map(oracle_map, device, pick(torch.int32, torch.int64))
+        device_generator = torch.Generator(device=device).manual_seed(seed)
+
+        def normal(*shape):
+            return torch.empty(shape, dtype=dtype, device=device).normal_(0, 0.5, generator=device_generator)
+
+        x = normal(oracle_map.num_rows, inner)
+        x[~oracle_map.real_row_mask().to(device)] = 0
+        case = f"seed {seed}: {experts} experts, inner {inner}, other {other}, {dtype}, {oracle_map.num_rows} rows"
+        weight = normal(experts * other, inner)
+        out = output_sparse_matmul(x, weight.t(), sparse_map)
+        expected = moe_oracle.output_sparse_matmul(x.float(), weight.t().float(), oracle_map)
+        assert max_rel_err(out, expected) <= _MAX_REL[dtype], case
+        weight = normal(experts * inner, other)
+        out = input_inner_sparse_matmul(x, weight, sparse_map)
+        expected = moe_oracle.input_inner_sparse_matmul(x.float(), weight.float(), oracle_map)
+        assert max_rel_err(out, expected) <= _MAX_REL[dtype], case
+        y = normal(oracle_map.num_rows, other)
+        out = input_row_sparse_matmul(x.t(), y, sparse_map)
+        expected = moe_oracle.input_row_sparse_matmul(x.t().float(), y.float(), oracle_map)
+        assert max_rel_err(out, expected) <= _MAX_REL[dtype], case
