@@ -233,12 +233,14 @@ struct TileLoader {
         // are 16 further on: 32 K-rows, eight times the four K-rows of `pair_stride`.
         const uint32_t lane_offset =
             offset[j & 1] + static_cast<uint32_t>(kHalves ? ((j >> 1) & 1) + 8 * (j >> 2) : j >> 1) * pair_stride;
-        const int block_address = __builtin_amdgcn_readfirstlane(slot_address + block_of(wave_index, j) * 1024);
+        // M0 = slot + the wavefront's part of the block number + the load's part: the last addition is made into M0
+        // itself, with the load's part as an immediate (one scalar instruction per load instead of two).
+        const int wave_address = __builtin_amdgcn_readfirstlane(slot_address + block_of(wave_index, 0) * 1024);
         // M0 is not handed out by the register allocator and nothing else in this file uses it.
-        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+        asm volatile("s_add_i32 m0, %0, %3\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      :
-                     : "s"(block_address), "v"(lane_offset), "s"(resource)
-                     : "memory");
+                     : "s"(wave_address), "v"(lane_offset), "s"(resource), "n"((block_of(0, j) - block_of(0, 0)) * 1024)
+                     : "memory", "scc");
     }
 };
 
